@@ -1,0 +1,334 @@
+// AdamW step kernels for gfx950: a flat single-tensor step and a
+// multi-tensor step that updates a whole parameter set in one launch.
+//
+// Arithmetic follows the reference kernel's operation order
+// (src/optimizer/adamw.cu:45-59, amsgrad :72-89): math in float (double for
+// double storage), m and v stored back in the storage type while the update
+// continues from the unrounded values, bias corrections formed on the host in
+// double and narrowed (adamw.cu:116-117).
+//
+// The op moves 28 B per fp32 parameter (read w, g, m, v; write w, m, v) and
+// does ~20 flops, so it is bound by HBM: every lane moves 16 B per access,
+// each workgroup owns one contiguous chunk, and nothing is read twice.
+#include "common.cuh"
+
+#include <math.h>
+
+namespace cs_hip {
+namespace {
+
+template <typename U>
+struct AdamHyper {
+  U lr, beta1, beta2, inv_bc1, inv_bc2, eps, wd;
+};
+
+template <typename U>
+__device__ __forceinline__ U dev_sqrt(U x);
+template <>
+__device__ __forceinline__ float dev_sqrt<float>(float x) {
+  return sqrtf(x);
+}
+template <>
+__device__ __forceinline__ double dev_sqrt<double>(double x) {
+  return sqrt(x);
+}
+
+// One element, reference operation order.
+template <typename T, bool AMSGRAD>
+__device__ __forceinline__ void adam_update(T &w, T &m, T &v, T &vmax, const T g_in,
+                                            const AdamHyper<typename Acc<T>::type> &h) {
+  using U = typename Acc<T>::type;
+  const U one = (U)1;
+  const U g = to_acc(g_in);
+  const U w0 = to_acc(w);
+  const U theta = w0 - h.lr * h.wd * w0;
+  const U m_t = h.beta1 * to_acc(m) + (one - h.beta1) * g;
+  m = from_acc<T>(m_t);
+  const U v_t = h.beta2 * to_acc(v) + (one - h.beta2) * g * g;
+  v = from_acc<T>(v_t);
+  const U m_hat = m_t * h.inv_bc1;
+  U v_hat = v_t * h.inv_bc2;
+  if constexpr (AMSGRAD) {
+    const U vm = to_acc(vmax);
+    v_hat = vm > v_hat ? vm : v_hat;
+    vmax = from_acc<T>(v_hat);
+  }
+  w = from_acc<T>(theta - h.lr * m_hat / (dev_sqrt<U>(v_hat) + h.eps));
+}
+
+constexpr int kAdamThreads = 256;
+constexpr int kAdamUnroll = 4;  // 16-byte vectors per lane per chunk
+
+template <typename T>
+constexpr int64_t adam_chunk_elems() {
+  return (int64_t)kAdamThreads * kAdamUnroll * Vec16<T>::n;
+}
+
+// Updates elements [begin, end) of one tensor with this workgroup.  `vec_ok`
+// says all five pointers are 16-byte aligned at element 0.
+template <typename T, bool AMSGRAD>
+__device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restrict__ dw,
+                                           T *__restrict__ m, T *__restrict__ v,
+                                           T *__restrict__ vmax, int64_t begin, int64_t end,
+                                           bool vec_ok,
+                                           const AdamHyper<typename Acc<T>::type> &h) {
+  constexpr int VN = Vec16<T>::n;
+  const int tid = threadIdx.x;
+  if (vec_ok && end - begin == adam_chunk_elems<T>()) {
+    // full chunk: issue every load before the first use
+    Vec16<T> vw[kAdamUnroll], vg[kAdamUnroll], vm[kAdamUnroll], vv[kAdamUnroll], vx[kAdamUnroll];
+#pragma unroll
+    for (int u = 0; u < kAdamUnroll; ++u) {
+      const int64_t off = begin + ((int64_t)u * kAdamThreads + tid) * VN;
+      vg[u] = load16_stream(dw + off);
+      vw[u] = load16_stream(w + off);
+      vm[u] = load16_stream(m + off);
+      vv[u] = load16_stream(v + off);
+      if constexpr (AMSGRAD) vx[u] = load16_stream(vmax + off);
+    }
+#pragma unroll
+    for (int u = 0; u < kAdamUnroll; ++u) {
+      const int64_t off = begin + ((int64_t)u * kAdamThreads + tid) * VN;
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        adam_update<T, AMSGRAD>(vw[u].e[k], vm[u].e[k], vv[u].e[k], vx[u].e[k], vg[u].e[k], h);
+      }
+      store16_stream(w + off, vw[u]);
+      store16_stream(m + off, vm[u]);
+      store16_stream(v + off, vv[u]);
+      if constexpr (AMSGRAD) store16_stream(vmax + off, vx[u]);
+    }
+    return;
+  }
+  // ragged chunk (tensor tail, small tensors, or unaligned pointers)
+  for (int64_t i = begin + tid; i < end; i += kAdamThreads) {
+    T wi = w[i], mi = m[i], vi = v[i], xi{};
+    if constexpr (AMSGRAD) xi = vmax[i];
+    adam_update<T, AMSGRAD>(wi, mi, vi, xi, dw[i], h);
+    w[i] = wi;
+    m[i] = mi;
+    v[i] = vi;
+    if constexpr (AMSGRAD) vmax[i] = xi;
+  }
+}
+
+template <typename T, bool AMSGRAD>
+__global__ __launch_bounds__(kAdamThreads) void adamw_flat_kernel(
+    T *__restrict__ w, const T *__restrict__ dw, T *__restrict__ m, T *__restrict__ v,
+    T *__restrict__ vmax, int64_t n, bool vec_ok, AdamHyper<typename Acc<T>::type> h) {
+  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t begin = (int64_t)blockIdx.x * chunk;
+  const int64_t end = begin + chunk < n ? begin + chunk : n;
+  adam_chunk<T, AMSGRAD>(w, dw, m, v, vmax, begin, end, vec_ok, h);
+}
+
+// ---------------------------------------------------------- multi-tensor
+// Device table: int64 first_slot[n_tensors + 1] (padded to a multiple of 8
+// entries), then one DevTensor per tensor.  Workgroup slot s belongs to the
+// tensor i with first_slot[i] <= s < first_slot[i+1] and updates that
+// tensor's chunk number s - first_slot[i].
+struct DevTensor {
+  void *w;
+  const void *dw;
+  void *m;
+  void *v;
+  void *vmax;
+  int64_t n;
+  int64_t vec_ok;
+  int64_t pad;
+};
+static_assert(sizeof(DevTensor) == 64, "table layout");
+
+__host__ __device__ inline int64_t slot_array_len(int64_t n_tensors) {
+  return (n_tensors + 1 + 7) / 8 * 8;
+}
+
+template <typename T, bool AMSGRAD>
+__global__ __launch_bounds__(kAdamThreads) void adamw_multi_kernel(
+    const int64_t *__restrict__ table, int n_tensors, AdamHyper<typename Acc<T>::type> h) {
+  const int64_t slot = blockIdx.x;
+  // binary search over the prefix array; wave-uniform, so it runs on the
+  // scalar unit out of the constant cache
+  int lo = 0, hi = n_tensors;  // invariant: first_slot[lo] <= slot < first_slot[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (table[mid] <= slot) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  const DevTensor *desc =
+      reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
+  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t begin = (slot - table[lo]) * chunk;
+  const int64_t n = desc->n;
+  const int64_t end = begin + chunk < n ? begin + chunk : n;
+  adam_chunk<T, AMSGRAD>(static_cast<T *>(desc->w), static_cast<const T *>(desc->dw),
+                         static_cast<T *>(desc->m), static_cast<T *>(desc->v),
+                         static_cast<T *>(desc->vmax), begin, end, desc->vec_ok != 0, h);
+}
+
+template <typename U>
+AdamHyper<U> make_hyper(double lr, double beta1, double beta2, double eps, double wd, int64_t t) {
+  AdamHyper<U> h;
+  h.lr = (U)lr;
+  h.beta1 = (U)beta1;
+  h.beta2 = (U)beta2;
+  // host double, then narrowed: adamw.cu:116-117
+  h.inv_bc1 = (U)(1. / (1. - pow(beta1, (double)t)));
+  h.inv_bc2 = (U)(1. / (1. - pow(beta2, (double)t)));
+  h.eps = (U)eps;
+  h.wd = (U)wd;
+  return h;
+}
+
+template <typename T>
+int64_t chunks_for(int64_t n) {
+  return ceil_div(n, adam_chunk_elems<T>());
+}
+
+int64_t chunks_for_dtype(int dtype, int64_t n) {
+  switch (dtype) {
+    case CS_F32: return chunks_for<float>(n);
+    case CS_F64: return chunks_for<double>(n);
+    case CS_F16: return chunks_for<f16_t>(n);
+    case CS_BF16: return chunks_for<bf16_t>(n);
+    default: return -1;
+  }
+}
+
+template <typename T>
+int launch_flat(void *w, const void *dw, void *m, void *v, void *vmax, int64_t n, double lr,
+                double beta1, double beta2, double eps, double wd, int64_t t, hipStream_t s) {
+  using U = typename Acc<T>::type;
+  const int64_t blocks = chunks_for<T>(n);
+  if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  const bool vec_ok = is_aligned16(w) && is_aligned16(dw) && is_aligned16(m) && is_aligned16(v) &&
+                      (vmax == nullptr || is_aligned16(vmax));
+  const AdamHyper<U> h = make_hyper<U>(lr, beta1, beta2, eps, wd, t);
+  if (vmax) {
+    adamw_flat_kernel<T, true><<<dim3((unsigned)blocks), dim3(kAdamThreads), 0, s>>>(
+        (T *)w, (const T *)dw, (T *)m, (T *)v, (T *)vmax, n, vec_ok, h);
+  } else {
+    adamw_flat_kernel<T, false><<<dim3((unsigned)blocks), dim3(kAdamThreads), 0, s>>>(
+        (T *)w, (const T *)dw, (T *)m, (T *)v, nullptr, n, vec_ok, h);
+  }
+  return launch_status();
+}
+
+template <typename T>
+int launch_multi(const void *table, int64_t n_tensors, int64_t n_slots, int amsgrad, double lr,
+                 double beta1, double beta2, double eps, double wd, int64_t t, hipStream_t s) {
+  using U = typename Acc<T>::type;
+  const AdamHyper<U> h = make_hyper<U>(lr, beta1, beta2, eps, wd, t);
+  const int64_t *tab = static_cast<const int64_t *>(table);
+  if (amsgrad) {
+    adamw_multi_kernel<T, true>
+        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h);
+  } else {
+    adamw_multi_kernel<T, false>
+        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h);
+  }
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace cs_hip
+
+using namespace cs_hip;
+
+extern "C" int cs_adamw_step(void *w, const void *dw, void *m, void *v, void *v_max, int64_t n,
+                             int dtype, double lr, double beta1, double beta2, double eps,
+                             double weight_decay, int64_t t, void *stream) {
+  if (n < 0) return CS_ERR_INVALID_ARGUMENT;
+  const size_t es = dtype_size(dtype);
+  if (es == 0) return CS_ERR_UNSUPPORTED;
+  if (n == 0) return CS_OK;
+  if (!w || !dw || !m || !v) return CS_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(w, es) || !aligned_to(dw, es) || !aligned_to(m, es) || !aligned_to(v, es) ||
+      (v_max && !aligned_to(v_max, es)))
+    return CS_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case CS_F32:
+      return launch_flat<float>(w, dw, m, v, v_max, n, lr, beta1, beta2, eps, weight_decay, t, s);
+    case CS_F64:
+      return launch_flat<double>(w, dw, m, v, v_max, n, lr, beta1, beta2, eps, weight_decay, t, s);
+    case CS_F16:
+      return launch_flat<f16_t>(w, dw, m, v, v_max, n, lr, beta1, beta2, eps, weight_decay, t, s);
+    case CS_BF16:
+      return launch_flat<bf16_t>(w, dw, m, v, v_max, n, lr, beta1, beta2, eps, weight_decay, t, s);
+  }
+  return CS_ERR_UNSUPPORTED;
+}
+
+extern "C" size_t cs_adamw_multi_table_bytes(int64_t n_tensors) {
+  if (n_tensors <= 0) return 0;
+  return (size_t)slot_array_len(n_tensors) * sizeof(int64_t) +
+         (size_t)n_tensors * sizeof(DevTensor);
+}
+
+// The chunk size depends on the element type, so a table is built for one
+// dtype and must be used with the same dtype in cs_adamw_multi_step.
+extern "C" int cs_adamw_multi_build_table(const cs_adamw_tensor *tensors, int64_t n_tensors,
+                                          int dtype, void *host_table, size_t table_bytes,
+                                          int64_t *n_slots) {
+  if (!tensors || !host_table || !n_slots || n_tensors <= 0) return CS_ERR_INVALID_ARGUMENT;
+  const size_t es = dtype_size(dtype);
+  if (es == 0) return CS_ERR_UNSUPPORTED;
+  if (table_bytes < cs_adamw_multi_table_bytes(n_tensors)) return CS_ERR_WORKSPACE;
+  int64_t *first_slot = static_cast<int64_t *>(host_table);
+  DevTensor *desc = reinterpret_cast<DevTensor *>(first_slot + slot_array_len(n_tensors));
+  int64_t slots = 0;
+  for (int64_t i = 0; i < n_tensors; ++i) {
+    const cs_adamw_tensor &t = tensors[i];
+    if (t.n < 0) return CS_ERR_INVALID_ARGUMENT;
+    if (t.n > 0) {
+      if (!t.w || !t.dw || !t.m || !t.v) return CS_ERR_INVALID_ARGUMENT;
+      if (!aligned_to(t.w, es) || !aligned_to(t.dw, es) || !aligned_to(t.m, es) ||
+          !aligned_to(t.v, es) || (t.v_max && !aligned_to(t.v_max, es)))
+        return CS_ERR_MISALIGNED;
+    }
+    first_slot[i] = slots;
+    desc[i].w = t.w;
+    desc[i].dw = t.dw;
+    desc[i].m = t.m;
+    desc[i].v = t.v;
+    desc[i].vmax = t.v_max;
+    desc[i].n = t.n;
+    desc[i].vec_ok = is_aligned16(t.w) && is_aligned16(t.dw) && is_aligned16(t.m) &&
+                     is_aligned16(t.v) && (t.v_max == nullptr || is_aligned16(t.v_max));
+    desc[i].pad = 0;
+    slots += chunks_for_dtype(dtype, t.n);
+  }
+  for (int64_t i = n_tensors; i < slot_array_len(n_tensors); ++i) first_slot[i] = slots;
+  if (slots > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  *n_slots = slots;
+  return CS_OK;
+}
+
+extern "C" int cs_adamw_multi_step(const void *device_table, int64_t n_tensors, int64_t n_slots,
+                                   int dtype, int amsgrad, double lr, double beta1, double beta2,
+                                   double eps, double weight_decay, int64_t t, void *stream) {
+  if (n_tensors < 0 || n_slots < 0) return CS_ERR_INVALID_ARGUMENT;
+  if (n_tensors == 0 || n_slots == 0) return CS_OK;
+  if (!device_table || !aligned_to(device_table, 16)) return CS_ERR_INVALID_ARGUMENT;
+  if (n_slots > 0x7fffffffLL || n_tensors > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case CS_F32:
+      return launch_multi<float>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
+                                 weight_decay, t, s);
+    case CS_F64:
+      return launch_multi<double>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
+                                  weight_decay, t, s);
+    case CS_F16:
+      return launch_multi<f16_t>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
+                                 weight_decay, t, s);
+    case CS_BF16:
+      return launch_multi<bf16_t>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
+                                  weight_decay, t, s);
+  }
+  return CS_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,357 @@
+// Fused classifier for gfx950: row softmax + cross-entropy loss + dlogits in
+// one pass over the logits.
+//
+// Replaces at::log_softmax + at::nll_loss_forward
+// (src/compute/cross_entropy.cpp:57-63) and at::nll_loss_backward +
+// at::_log_softmax_backward_data (:103-109), which between them make about
+// five passes over [N, V] and keep three [N, V] temporaries:
+//   loss_i    = logsumexp(x_i) - x_i[t_i]            (0 for ignored rows)
+//   loss      = sum_i loss_i / #{not ignored}        (MEAN)  |  sum_i loss_i (SUM)
+//   dlogits_i = (softmax(x_i) - onehot(t_i)) * s,    s = dloss / #{not ignored} (MEAN) | dloss
+//
+// One workgroup owns one row and keeps it in registers as 16-byte vectors
+// (50257 bf16 = 6283 vectors = 7 per lane at 1024 lanes, 28 VGPRs), so the
+// row is read from HBM once and dlogits written once: 2 accesses per
+// element.  The max and the sum of exponentials are exact two-step
+// reductions over registers (wave64 butterfly, then LDS across the 16
+// waves), not a running rescale; the probabilities are formed as
+// 2^(x*log2e - K) with K = max*log2e + log2(sum) - log2(s) folded into one
+// constant, which costs one fma and one hardware exp2 per element.
+#include "common.cuh"
+
+#include <math.h>
+
+#include <type_traits>
+
+namespace cs_hip {
+namespace {
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kLn2 = 0.69314718055994530942f;
+
+// workspace: [0] int32 count of rows not ignored, [1] float the same number,
+// then (from byte 256) N floats of row loss when the caller keeps none.
+constexpr size_t kWsHeader = 256;
+
+__device__ __forceinline__ bool target_counts(int64_t t, int64_t V, int64_t ignore_index) {
+  return t != ignore_index && t >= 0 && t < V;
+}
+
+__global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t *__restrict__ targets,
+                                                        int64_t N, int64_t V,
+                                                        int64_t ignore_index,
+                                                        int *__restrict__ ws_count,
+                                                        float *__restrict__ ws_weight) {
+  __shared__ int scratch[16];
+  int c = 0;
+  for (int64_t i = threadIdx.x; i < N; i += 1024) c += target_counts(targets[i], V, ignore_index);
+  c = block_reduce(c, SumOp{}, 0, scratch);
+  if (threadIdx.x == 0) {
+    *ws_count = c;
+    *ws_weight = (float)c;
+  }
+}
+
+// Fixed-order sum of the row losses: thread t adds rows t, t+1024, ...; the
+// 1024 sub-sums are folded by the butterfly.  Independent of scheduling.
+__global__ __launch_bounds__(1024) void ce_reduce_kernel(const float *__restrict__ row_loss,
+                                                         int64_t N, const int *__restrict__ ws_count,
+                                                         int reduction, float *__restrict__ loss,
+                                                         float *__restrict__ total_weight) {
+  __shared__ float scratch[16];
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < N; i += 1024) s += row_loss[i];
+  s = block_reduce(s, SumOp{}, 0.f, scratch);
+  if (threadIdx.x == 0) {
+    const int c = *ws_count;
+    if (loss) *loss = reduction == CS_REDUCTION_MEAN ? s / (float)c : s;
+    if (total_weight) *total_weight = (float)c;
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ float vec_get(const Vec16<T> &v, int k) {
+  return to_acc(v.e[k]);
+}
+
+// TD is the dlogits storage: T, or float when the caller wants fp32 gradients
+// for 16-bit logits.
+template <typename T, typename TD, int N_ELEMS>
+__device__ __forceinline__ void store_out(TD *p, const float (&o)[N_ELEMS]) {
+  constexpr int DN = Vec16<TD>::n;
+#pragma unroll
+  for (int q = 0; q < N_ELEMS / DN; ++q) {
+    Vec16<TD> v;
+#pragma unroll
+    for (int k = 0; k < DN; ++k) v.e[k] = from_acc<TD>(o[q * DN + k]);
+    store16_stream(p + q * DN, v);
+  }
+}
+
+template <typename T, typename TD, int BLOCK, int VPT>
+__global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
+    const T *__restrict__ logits, TD *__restrict__ dlogits, const int64_t *__restrict__ targets,
+    float *__restrict__ row_loss, const int *__restrict__ ws_count, int64_t V, int64_t row_stride,
+    int64_t ignore_index, int reduction, float dloss) {
+  constexpr int VN = Vec16<T>::n;
+  __shared__ float scratch[(BLOCK + kWave - 1) / kWave];
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int nvec = (int)(row_stride / VN);  // whole row incl. padding, in vectors
+  const int iV = (int)V;
+  const T *x = logits + row * row_stride;
+  const int64_t target = targets[row];
+  const bool counts = target_counts(target, V, ignore_index);  // block-uniform
+
+  if (!counts) {
+    if (tid == 0 && row_loss) row_loss[row] = 0.f;
+    if (dlogits) {
+      float z[VN];
+#pragma unroll
+      for (int k = 0; k < VN; ++k) z[k] = 0.f;
+      for (int idx = tid; idx < nvec; idx += BLOCK)
+        store_out<T, TD, VN>(dlogits + row * row_stride + (int64_t)idx * VN, z);
+    }
+    return;
+  }
+
+  Vec16<T> xr[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int idx = tid + BLOCK * j;
+    if (idx < nvec) xr[j] = load16_stream(x + (int64_t)idx * VN);
+  }
+  const float x_t = tid == 0 ? to_acc(x[target]) : 0.f;
+
+  // ---- row maximum
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (tid + BLOCK * j) * VN;
+    if (c0 + VN <= iV) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) m = fmaxf(m, vec_get(xr[j], k));
+    } else if (c0 < iV) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k)
+        if (c0 + k < iV) m = fmaxf(m, vec_get(xr[j], k));
+    }
+  }
+  m = block_reduce(m, MaxOp{}, -INFINITY, scratch);
+  const float m2 = m * kLog2e;
+
+  // ---- sum of exponentials
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (tid + BLOCK * j) * VN;
+    if (c0 + VN <= iV) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) s += __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - m2);
+    } else if (c0 < iV) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k)
+        if (c0 + k < iV) s += __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - m2);
+    }
+  }
+  s = block_reduce(s, SumOp{}, 0.f, scratch);
+
+  const float log2_s = __builtin_amdgcn_logf(s);  // v_log_f32 is log2
+  if (tid == 0 && row_loss) row_loss[row] = (m2 + log2_s) * kLn2 - x_t;
+  if (dlogits == nullptr) return;
+
+  // ---- dlogits = (p - onehot) * scale, p * scale = 2^(x*log2e - K)
+  float scale = dloss;
+  if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
+  // K folds max, sum and |scale|; the sign of scale is applied afterwards
+  const float abs_scale = fabsf(scale);
+  const float K = m2 + log2_s - __builtin_amdgcn_logf(abs_scale);
+  const float sign = scale < 0.f ? -1.f : 1.f;
+  const int t_vec = (int)(target / VN), t_sub = (int)(target % VN);
+  TD *d = dlogits + row * row_stride;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int idx = tid + BLOCK * j;
+    if (idx < nvec) {
+      const int c0 = idx * VN;
+      float o[VN];
+      if (abs_scale == 0.f) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) o[k] = 0.f;
+      } else {
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          o[k] = sign * __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - K);
+      }
+      if (c0 + VN > iV) {  // last class vector and the padding
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          if (c0 + k >= iV) o[k] = 0.f;
+      }
+      if (idx == t_vec) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          if (k == t_sub) o[k] -= scale;
+      }
+      store_out<T, TD, VN>(d + (int64_t)c0, o);
+    }
+  }
+}
+
+// Any V, stride and alignment; fp64 too.  Three sweeps over the row, the
+// later ones served by the cache.
+template <typename T, typename TD>
+__global__ __launch_bounds__(256) void ce_rows_general_kernel(
+    const T *__restrict__ logits, TD *__restrict__ dlogits, const int64_t *__restrict__ targets,
+    float *__restrict__ row_loss, const int *__restrict__ ws_count, int64_t V, int64_t row_stride,
+    int64_t ignore_index, int reduction, float dloss) {
+  using U = typename Acc<T>::type;
+  __shared__ U scratch[4];
+  const int64_t row = blockIdx.x;
+  const T *x = logits + row * row_stride;
+  const int64_t target = targets[row];
+  const bool counts = target_counts(target, V, ignore_index);
+  if (!counts) {
+    if (threadIdx.x == 0 && row_loss) row_loss[row] = 0.f;
+    if (dlogits)
+      for (int64_t c = threadIdx.x; c < row_stride; c += 256)
+        dlogits[row * row_stride + c] = from_acc<TD>((typename Acc<TD>::type)0);
+    return;
+  }
+  U m = -INFINITY;
+  for (int64_t c = threadIdx.x; c < V; c += 256) {
+    const U v = to_acc(x[c]);
+    m = v > m ? v : m;
+  }
+  m = block_reduce(m, MaxOp{}, (U)-INFINITY, scratch);
+  U s = 0;
+  for (int64_t c = threadIdx.x; c < V; c += 256) s += exp((U)to_acc(x[c]) - m);
+  s = block_reduce(s, SumOp{}, (U)0, scratch);
+  const U lse = m + log(s);
+  if (threadIdx.x == 0 && row_loss) row_loss[row] = (float)(lse - (U)to_acc(x[target]));
+  if (!dlogits) return;
+  U scale = (U)dloss;
+  if (reduction == CS_REDUCTION_MEAN) scale = (U)dloss / (U)(*ws_count);
+  for (int64_t c = threadIdx.x; c < row_stride; c += 256) {
+    U o = 0;
+    if (c < V) {
+      o = exp((U)to_acc(x[c]) - lse);
+      if (c == target) o -= (U)1;
+      o *= scale;
+    }
+    dlogits[row * row_stride + c] = from_acc<TD>((typename Acc<TD>::type)o);
+  }
+}
+
+template <typename T, typename TD>
+int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
+                const int *ws_count, int64_t N, int64_t V, int64_t row_stride,
+                int64_t ignore_index, int reduction, float dloss, hipStream_t s) {
+  constexpr int VN = Vec16<T>::n;
+  const bool vec_ok = !std::is_same_v<T, double> && row_stride % VN == 0 && is_aligned16(logits) &&
+                      (!dlogits || is_aligned16(dlogits)) && row_stride / VN <= 1024 * 16;
+  const dim3 grid((unsigned)N);
+  if constexpr (!std::is_same_v<T, double>) {
+    if (vec_ok) {
+      const int64_t nvec = row_stride / VN;
+#define CS_CE(BLOCK, VPT)                                                                   \
+  ce_rows_kernel<T, TD, BLOCK, VPT><<<grid, dim3(BLOCK), 0, s>>>(                           \
+      (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, V, row_stride,         \
+      ignore_index, reduction, dloss)
+      if (nvec <= 64 * 8) {
+        CS_CE(64, 8);
+      } else if (nvec <= 256 * 8) {
+        CS_CE(256, 8);
+      } else if (nvec <= 1024 * 7) {
+        CS_CE(1024, 7);
+      } else if (nvec <= 1024 * 8) {
+        CS_CE(1024, 8);
+      } else {
+        CS_CE(1024, 16);
+      }
+#undef CS_CE
+      return launch_status();
+    }
+  }
+  ce_rows_general_kernel<T, TD><<<grid, dim3(256), 0, s>>>((const T *)logits, (TD *)dlogits,
+                                                            targets, row_loss, ws_count, V,
+                                                            row_stride, ignore_index, reduction,
+                                                            dloss);
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace cs_hip
+
+using namespace cs_hip;
+
+extern "C" size_t cs_fused_classifier_workspace_bytes(int64_t N) {
+  if (N < 0) return 0;
+  return kWsHeader + ((size_t)N * sizeof(float) + 255) / 256 * 256;
+}
+
+extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int64_t *targets,
+                                   float *row_loss, float *loss, float *total_weight,
+                                   void *workspace, size_t workspace_bytes, int64_t N, int64_t V,
+                                   int64_t row_stride, int64_t ignore_index, int reduction,
+                                   float dloss, int dtype, int dlogits_dtype, void *stream) {
+  if (N < 0 || V <= 0 || row_stride < V) return CS_ERR_INVALID_ARGUMENT;
+  if (reduction != CS_REDUCTION_NONE && reduction != CS_REDUCTION_MEAN &&
+      reduction != CS_REDUCTION_SUM)
+    return CS_ERR_INVALID_ARGUMENT;
+  const size_t es = dtype_size(dtype), ds = dtype_size(dlogits_dtype);
+  if (es == 0 || ds == 0) return CS_ERR_UNSUPPORTED;
+  if (dlogits_dtype != dtype && !(dlogits_dtype == CS_F32 && es == 2)) return CS_ERR_UNSUPPORTED;
+  if (N > 0x7fffffffLL || V > 0x7fffffffLL || row_stride > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  if (!workspace || workspace_bytes < cs_fused_classifier_workspace_bytes(N) ||
+      !aligned_to(workspace, 256))
+    return CS_ERR_WORKSPACE;
+  if (reduction == CS_REDUCTION_NONE && !row_loss) return CS_ERR_INVALID_ARGUMENT;
+  if (reduction != CS_REDUCTION_NONE && !loss) return CS_ERR_INVALID_ARGUMENT;
+  if (N > 0 && (!logits || !targets)) return CS_ERR_INVALID_ARGUMENT;
+  if ((logits && !aligned_to(logits, es)) || (dlogits && !aligned_to(dlogits, ds)) ||
+      (targets && !aligned_to(targets, 8)) || (row_loss && !aligned_to(row_loss, 4)) ||
+      (loss && !aligned_to(loss, 4)) || (total_weight && !aligned_to(total_weight, 4)))
+    return CS_ERR_MISALIGNED;
+  if (dlogits == logits && dlogits_dtype != dtype) return CS_ERR_INVALID_ARGUMENT;
+
+  hipStream_t s = as_stream(stream);
+  char *ws = static_cast<char *>(workspace);
+  int *ws_count = reinterpret_cast<int *>(ws);
+  float *ws_weight = reinterpret_cast<float *>(ws) + 1;
+  float *rows = row_loss ? row_loss : reinterpret_cast<float *>(ws + kWsHeader);
+
+  ce_count_kernel<<<dim3(1), dim3(1024), 0, s>>>(targets, N, V, ignore_index, ws_count, ws_weight);
+  int st = launch_status();
+  if (st != CS_OK) return st;
+  if (N > 0) {
+#define CS_CALL(T, TD)                                                                     \
+  st = launch_rows<T, TD>(logits, dlogits, targets, rows, ws_count, N, V, row_stride,      \
+                          ignore_index, reduction, dloss, s)
+    const bool wide = dlogits_dtype != dtype;
+    switch (dtype) {
+      case CS_F32: CS_CALL(float, float); break;
+      case CS_F64: CS_CALL(double, double); break;
+      case CS_F16:
+        if (wide) {
+          CS_CALL(f16_t, float);
+        } else {
+          CS_CALL(f16_t, f16_t);
+        }
+        break;
+      case CS_BF16:
+        if (wide) {
+          CS_CALL(bf16_t, float);
+        } else {
+          CS_CALL(bf16_t, bf16_t);
+        }
+        break;
+    }
+#undef CS_CALL
+    if (st != CS_OK) return st;
+  }
+  ce_reduce_kernel<<<dim3(1), dim3(1024), 0, s>>>(rows, N, ws_count, reduction,
+                                                  reduction == CS_REDUCTION_NONE ? nullptr : loss,
+                                                  total_weight);
+  return launch_status();
+}

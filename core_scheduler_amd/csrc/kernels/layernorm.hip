@@ -1,0 +1,652 @@
+// LayerNorm forward / backward over the last dimension for gfx950.
+//
+// Replaces at::native_layer_norm (src/compute/layer_norm.cpp:163-169,
+// :198-204) and the two at::native_layer_norm_backward calls (:263-266 for
+// dx, :321-334 / :375-383 for dgamma and dbeta).  Statistics and all
+// arithmetic are fp32 for f32/f16/bf16 storage (fp64 for f64):
+//   mean = sum(x)/C, var = sum((x-mean)^2)/C (biased), rstd = 1/sqrt(var+eps)
+//   y    = (x-mean)*rstd*gamma + beta
+//   dx   = rstd * (g - mean_C(g) - xhat*mean_C(g*xhat)),  g = dy*gamma
+//   dgamma = sum_rows(dy*xhat), dbeta = sum_rows(dy)
+//
+// Fast path: one wavefront owns whole rows.  A row lives in registers as
+// 16-byte vectors (lane l holds vectors l, l+64, ...), the two row sums are
+// wave64 butterflies, and nothing is read twice: forward moves x once in and
+// y once out, backward reads dy and x once and produces dx and the
+// per-column partial sums in the same pass.  Each lane keeps the partial
+// dgamma/dbeta of its own columns in registers across all rows its wave
+// visits; a workgroup folds its waves through LDS and writes one partial row
+// per workgroup, and a second small kernel adds the partial rows in a fixed
+// order, so the result does not depend on scheduling and uses no atomics.
+//
+// Anything the fast path cannot take (C not a multiple of the vector width,
+// C beyond the register budget, unaligned pointers, fp64) goes through a
+// plain one-workgroup-per-row path.
+#include "common.cuh"
+
+#include <math.h>
+
+#include <type_traits>
+
+namespace cs_hip {
+namespace {
+
+// ------------------------------------------------------------ n-wide access
+// N consecutive elements of T (N * sizeof(T) is 16 or 32 bytes) <-> fp32.
+template <typename T, int N>
+__device__ __forceinline__ void load_n(const T *p, float (&out)[N]) {
+  constexpr int VN = Vec16<T>::n;
+  static_assert(N % VN == 0, "whole 16-byte pieces");
+#pragma unroll
+  for (int q = 0; q < N / VN; ++q) {
+    const Vec16<T> v = load16(p + q * VN);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) out[q * VN + k] = to_acc(v.e[k]);
+  }
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_n(T *p, const float (&in)[N]) {
+  constexpr int VN = Vec16<T>::n;
+  static_assert(N % VN == 0, "whole 16-byte pieces");
+#pragma unroll
+  for (int q = 0; q < N / VN; ++q) {
+    Vec16<T> v;
+#pragma unroll
+    for (int k = 0; k < VN; ++k) v.e[k] = from_acc<T>(in[q * VN + k]);
+    store16_stream(p + q * VN, v);
+  }
+}
+// raw (still packed) row pieces, so a row costs 4 VGPRs per 16 bytes
+template <typename T, int N>
+struct Raw {
+  Vec16<T> v[N / Vec16<T>::n];
+};
+template <typename T, int N>
+__device__ __forceinline__ Raw<T, N> load_raw(const T *p) {
+  Raw<T, N> r;
+#pragma unroll
+  for (int q = 0; q < N / Vec16<T>::n; ++q) r.v[q] = load16_stream(p + q * Vec16<T>::n);
+  return r;
+}
+template <typename T, int N>
+__device__ __forceinline__ Raw<T, N> zero_raw() {
+  Raw<T, N> r;
+#pragma unroll
+  for (int q = 0; q < N / Vec16<T>::n; ++q)
+#pragma unroll
+    for (int k = 0; k < Vec16<T>::n; ++k) r.v[q].e[k] = T{};
+  return r;
+}
+template <typename T, int N>
+__device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
+  return to_acc(r.v[i / Vec16<T>::n].e[i % Vec16<T>::n]);
+}
+
+constexpr int kLnThreads = 256;  // 4 waves
+
+// ------------------------------------------------------------ fast forward
+// VPL: 16-byte x vectors per lane; R: rows per wave.
+template <typename TX, typename TY, typename TP, int VPL, int R>
+__global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
+    const TX *__restrict__ x, const TP *__restrict__ gamma, const TP *__restrict__ beta,
+    TY *__restrict__ y, float *__restrict__ mean, float *__restrict__ rstd, int64_t rows, int C,
+    float eps) {
+  constexpr int VN = Vec16<TX>::n;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t gw = (int64_t)blockIdx.x * (kLnThreads / kWave) + (threadIdx.x >> 6);
+  const int64_t row0 = gw * R;
+  if (row0 >= rows) return;  // wave-uniform
+  const int nvec = C / VN;
+
+  Raw<TX, VN> xr[R][VPL];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int idx = lane + kWave * j;
+      if (idx < nvec && row0 + r < rows) {
+        xr[r][j] = load_raw<TX, VN>(x + (row0 + r) * C + (int64_t)idx * VN);
+      } else {
+        xr[r][j] = zero_raw<TX, VN>();
+      }
+    }
+  }
+  float g[VPL][VN], b[VPL][VN];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int idx = lane + kWave * j;
+    if (idx < nvec) {
+      load_n<TP, VN>(gamma + idx * VN, g[j]);
+      if (beta) {
+        load_n<TP, VN>(beta + idx * VN, b[j]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) b[j][k] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        g[j][k] = 0.f;
+        b[j][k] = 0.f;
+      }
+    }
+  }
+  const float inv_c = 1.0f / (float)C;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (row0 + r >= rows) break;
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+#pragma unroll
+      for (int k = 0; k < VN; ++k) s += raw_get<TX, VN>(xr[r][j], k);
+    const float mu = wave_reduce(s, SumOp{}) * inv_c;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      if (lane + kWave * j < nvec) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          const float d = raw_get<TX, VN>(xr[r][j], k) - mu;
+          q += d * d;
+        }
+      }
+    }
+    const float var = wave_reduce(q, SumOp{}) * inv_c;
+    const float rs = 1.0f / sqrtf(var + eps);
+    if (lane == 0) {
+      mean[row0 + r] = mu;
+      rstd[row0 + r] = rs;
+    }
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int idx = lane + kWave * j;
+      if (idx < nvec) {
+        float o[VN];
+#pragma unroll
+        for (int k = 0; k < VN; ++k)
+          o[k] = (raw_get<TX, VN>(xr[r][j], k) - mu) * rs * g[j][k] + b[j][k];
+        store_n<TY, VN>(y + (row0 + r) * C + (int64_t)idx * VN, o);
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------- fast backward
+template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int R, bool HAS_DX,
+          bool HAS_DP>
+__global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
+    const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
+    const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
+    float *__restrict__ partial, int64_t rows, int C) {
+  constexpr int VN = Vec16<TX>::n;
+  extern __shared__ float lds[];  // [waves per block][C]
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  constexpr int kWaves = kLnThreads / kWave;
+  const int64_t gw = (int64_t)blockIdx.x * kWaves + wave;
+  const int64_t n_waves = (int64_t)gridDim.x * kWaves;
+  const int nvec = C / VN;
+  const float inv_c = 1.0f / (float)C;
+
+  float acc_g[VPL][VN], acc_b[VPL][VN], g[VPL][VN];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      acc_g[j][k] = 0.f;
+      acc_b[j][k] = 0.f;
+      g[j][k] = 0.f;
+    }
+    if (HAS_DX && lane + kWave * j < nvec) load_n<TP, VN>(gamma + (lane + kWave * j) * VN, g[j]);
+  }
+
+  for (int64_t row0 = gw * R; row0 < rows; row0 += n_waves * R) {
+    Raw<TDY, VN> dr[R][VPL];
+    Raw<TX, VN> xr[R][VPL];
+    float mu[R], rs[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bool live = row0 + r < rows;
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int idx = lane + kWave * j;
+        if (live && idx < nvec) {
+          const int64_t off = (row0 + r) * C + (int64_t)idx * VN;
+          dr[r][j] = load_raw<TDY, VN>(dy + off);
+          xr[r][j] = load_raw<TX, VN>(x + off);
+        } else {
+          dr[r][j] = zero_raw<TDY, VN>();
+          xr[r][j] = zero_raw<TX, VN>();
+        }
+      }
+      mu[r] = live ? mean[row0 + r] : 0.f;
+      rs[r] = live ? rstd[row0 + r] : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (row0 + r >= rows) break;
+      float s1 = 0.f, s2 = 0.f;
+      float xh[VPL][VN], dv[VPL][VN];
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          // lanes past the row hold zeros in dr, so they add nothing
+          xh[j][k] = (raw_get<TX, VN>(xr[r][j], k) - mu[r]) * rs[r];
+          dv[j][k] = raw_get<TDY, VN>(dr[r][j], k);
+          if constexpr (HAS_DP) {
+            acc_g[j][k] += dv[j][k] * xh[j][k];
+            acc_b[j][k] += dv[j][k];
+          }
+          if constexpr (HAS_DX) {
+            const float gd = dv[j][k] * g[j][k];
+            s1 += gd;
+            s2 += gd * xh[j][k];
+          }
+        }
+      }
+      if constexpr (HAS_DX) {
+        s1 = wave_reduce(s1, SumOp{}) * inv_c;
+        s2 = wave_reduce(s2, SumOp{}) * inv_c;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          const int idx = lane + kWave * j;
+          if (idx < nvec) {
+            float o[VN];
+#pragma unroll
+            for (int k = 0; k < VN; ++k)
+              o[k] = rs[r] * (dv[j][k] * g[j][k] - s1 - xh[j][k] * s2);
+            store_n<TDX, VN>(dx + (row0 + r) * C + (int64_t)idx * VN, o);
+          }
+        }
+      }
+    }
+  }
+
+  if constexpr (HAS_DP) {
+    // fold the block's waves, dgamma first, then dbeta through the same LDS
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int idx = lane + kWave * j;
+        if (idx < nvec) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            lds[wave * C + idx * VN + k] = which == 0 ? acc_g[j][k] : acc_b[j][k];
+        }
+      }
+      __syncthreads();
+      for (int c = threadIdx.x; c < C; c += kLnThreads) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) s += lds[w * C + c];
+        partial[((int64_t)blockIdx.x * 2 + which) * C + c] = s;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// Adds `nparts` partial rows in ascending order.  grid (ceil(C/64), 2),
+// block (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one
+// column, then row 0 of the block adds the 16 sub-sums in order.
+template <typename TP>
+__global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__restrict__ partial,
+                                                               int nparts, TP *__restrict__ dgamma,
+                                                               TP *__restrict__ dbeta, int C,
+                                                               int accumulate) {
+  __shared__ float sub[16][64];
+  const int which = blockIdx.y;
+  TP *out = which == 0 ? dgamma : dbeta;
+  if (out == nullptr) return;  // block-uniform
+  const int col = blockIdx.x * 64 + threadIdx.x;
+  float s = 0.f;
+  if (col < C) {
+    for (int p = threadIdx.y; p < nparts; p += 16) s += partial[((int64_t)p * 2 + which) * C + col];
+  }
+  sub[threadIdx.y][threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.y == 0 && col < C) {
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t += sub[r][threadIdx.x];
+    if (accumulate) t += to_acc(out[col]);
+    out[col] = from_acc<TP>(t);
+  }
+}
+
+// ------------------------------------------------------------ general path
+// One workgroup per row, any C, any alignment, fp64 included.
+template <typename TX, typename TY, typename TP>
+__global__ __launch_bounds__(kLnThreads) void ln_fwd_general_kernel(
+    const TX *__restrict__ x, const TP *__restrict__ gamma, const TP *__restrict__ beta,
+    TY *__restrict__ y, typename Acc<TX>::type *__restrict__ mean,
+    typename Acc<TX>::type *__restrict__ rstd, int64_t C, typename Acc<TX>::type eps) {
+  using U = typename Acc<TX>::type;
+  __shared__ U scratch[kLnThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const TX *xr = x + row * C;
+  U s = 0;
+  for (int64_t c = threadIdx.x; c < C; c += kLnThreads) s += to_acc(xr[c]);
+  const U mu = block_reduce(s, SumOp{}, (U)0, scratch) / (U)C;
+  U q = 0;
+  for (int64_t c = threadIdx.x; c < C; c += kLnThreads) {
+    const U d = to_acc(xr[c]) - mu;
+    q += d * d;
+  }
+  const U var = block_reduce(q, SumOp{}, (U)0, scratch) / (U)C;
+  const U rs = (U)1 / sqrt(var + eps);
+  if (threadIdx.x == 0) {
+    mean[row] = mu;
+    rstd[row] = rs;
+  }
+  for (int64_t c = threadIdx.x; c < C; c += kLnThreads) {
+    const U bb = beta ? (U)to_acc(beta[c]) : (U)0;
+    y[row * C + c] = from_acc<TY>((U)((to_acc(xr[c]) - mu) * rs * (U)to_acc(gamma[c]) + bb));
+  }
+}
+
+template <typename TDY, typename TX, typename TDX, typename TP>
+__global__ __launch_bounds__(kLnThreads) void ln_bwd_dx_general_kernel(
+    const TDY *__restrict__ dy, const TX *__restrict__ x,
+    const typename Acc<TX>::type *__restrict__ mean,
+    const typename Acc<TX>::type *__restrict__ rstd, const TP *__restrict__ gamma,
+    TDX *__restrict__ dx, int64_t C) {
+  using U = typename Acc<TX>::type;
+  __shared__ U scratch[kLnThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const U mu = mean[row], rs = rstd[row];
+  U s1 = 0, s2 = 0;
+  for (int64_t c = threadIdx.x; c < C; c += kLnThreads) {
+    const U gd = (U)to_acc(dy[row * C + c]) * (U)to_acc(gamma[c]);
+    const U xh = ((U)to_acc(x[row * C + c]) - mu) * rs;
+    s1 += gd;
+    s2 += gd * xh;
+  }
+  s1 = block_reduce(s1, SumOp{}, (U)0, scratch) / (U)C;
+  s2 = block_reduce(s2, SumOp{}, (U)0, scratch) / (U)C;
+  for (int64_t c = threadIdx.x; c < C; c += kLnThreads) {
+    const U gd = (U)to_acc(dy[row * C + c]) * (U)to_acc(gamma[c]);
+    const U xh = ((U)to_acc(x[row * C + c]) - mu) * rs;
+    dx[row * C + c] = from_acc<TDX>((U)(rs * (gd - s1 - xh * s2)));
+  }
+}
+
+// grid ceil(C/64) blocks of (64, 4): thread (cx, ry) walks rows ry, ry+4, ...
+template <typename TDY, typename TX, typename TP>
+__global__ __launch_bounds__(256) void ln_bwd_param_general_kernel(
+    const TDY *__restrict__ dy, const TX *__restrict__ x,
+    const typename Acc<TX>::type *__restrict__ mean,
+    const typename Acc<TX>::type *__restrict__ rstd, TP *__restrict__ dgamma,
+    TP *__restrict__ dbeta, int64_t rows, int64_t C, int accumulate) {
+  using U = typename Acc<TX>::type;
+  __shared__ U sg[4][64], sb[4][64];
+  const int64_t col = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  U ag = 0, ab = 0;
+  if (col < C) {
+    for (int64_t r = threadIdx.y; r < rows; r += 4) {
+      const U d = to_acc(dy[r * C + col]);
+      ag += d * (((U)to_acc(x[r * C + col]) - mean[r]) * rstd[r]);
+      ab += d;
+    }
+  }
+  sg[threadIdx.y][threadIdx.x] = ag;
+  sb[threadIdx.y][threadIdx.x] = ab;
+  __syncthreads();
+  if (threadIdx.y == 0 && col < C) {
+    U tg = 0, tb = 0;
+    for (int r = 0; r < 4; ++r) {
+      tg += sg[r][threadIdx.x];
+      tb += sb[r][threadIdx.x];
+    }
+    if (dgamma) {
+      if (accumulate) tg += (U)to_acc(dgamma[col]);
+      dgamma[col] = from_acc<TP>(tg);
+    }
+    if (dbeta) {
+      if (accumulate) tb += (U)to_acc(dbeta[col]);
+      dbeta[col] = from_acc<TP>(tb);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- dispatch
+struct FastPlan {
+  int vpl = 0;  // 0: not eligible
+  int rows_per_wave = 1;
+};
+
+// x vectors per lane needed for C columns of x_dtype; the fast kernels are
+// instantiated for 2, 4 and 8.
+FastPlan fast_plan(int64_t C, int x_dtype) {
+  FastPlan p;
+  const int vn = 16 / (int)dtype_size(x_dtype);
+  if (x_dtype == CS_F64 || C <= 0 || C % vn != 0) return p;
+  const int64_t nvec = C / vn;
+  const int64_t per_lane = ceil_div(nvec, (int64_t)kWave);
+  if (per_lane <= 2) {
+    p.vpl = 2;
+    p.rows_per_wave = 4;
+  } else if (per_lane <= 4) {
+    p.vpl = 4;
+    p.rows_per_wave = 2;
+  } else if (per_lane <= 8) {
+    p.vpl = 8;
+    p.rows_per_wave = 1;
+  }
+  return p;
+}
+
+constexpr int kLnBwdMaxBlocks = 1024;
+
+int ln_bwd_blocks(int64_t rows, const FastPlan &p) {
+  const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * p.rows_per_wave;
+  const int64_t b = ceil_div(rows, rows_per_block);
+  return (int)(b < kLnBwdMaxBlocks ? b : kLnBwdMaxBlocks);
+}
+
+template <typename TX, typename TY, typename TP>
+int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void *mean, void *rstd,
+              int64_t rows, int64_t C, double eps, bool aligned, int x_dtype, hipStream_t s) {
+  const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
+  if constexpr (!std::is_same_v<TX, double>) {
+    if (p.vpl != 0) {
+      const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * p.rows_per_wave;
+      const int64_t blocks = ceil_div(rows, rows_per_block);
+      if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+      const dim3 grid((unsigned)blocks), block(kLnThreads);
+#define CS_LN_FWD(VPL, R)                                                                   \
+  ln_fwd_rows_kernel<TX, TY, TP, VPL, R><<<grid, block, 0, s>>>(                            \
+      (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean,           \
+      (float *)rstd, rows, (int)C, (float)eps)
+      if (p.vpl == 2) {
+        CS_LN_FWD(2, 4);
+      } else if (p.vpl == 4) {
+        CS_LN_FWD(4, 2);
+      } else {
+        CS_LN_FWD(8, 1);
+      }
+#undef CS_LN_FWD
+      return launch_status();
+    }
+  }
+  using U = typename Acc<TX>::type;
+  if (rows > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  ln_fwd_general_kernel<TX, TY, TP><<<dim3((unsigned)rows), dim3(kLnThreads), 0, s>>>(
+      (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (U *)mean, (U *)rstd, C,
+      (U)eps);
+  return launch_status();
+}
+
+template <typename TDY, typename TX, typename TDX, typename TP>
+int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
+              const void *gamma, void *dx, void *dgamma, void *dbeta, void *workspace,
+              size_t workspace_bytes, int64_t rows, int64_t C, bool aligned, int x_dtype,
+              int accumulate, hipStream_t s) {
+  const bool want_dp = dgamma != nullptr || dbeta != nullptr;
+  const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
+  if constexpr (!std::is_same_v<TX, double>) {
+    if (p.vpl != 0) {
+      const int blocks = ln_bwd_blocks(rows, p);
+      const size_t need = want_dp ? (size_t)blocks * 2 * C * sizeof(float) : 0;
+      if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
+      const size_t lds = want_dp ? (size_t)(kLnThreads / kWave) * C * sizeof(float) : 0;
+      const dim3 grid((unsigned)blocks), block(kLnThreads);
+#define CS_LN_BWD(VPL, R, HAS_DX, HAS_DP)                                                   \
+  ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, R, HAS_DX, HAS_DP><<<grid, block, lds, s>>>(    \
+      (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd,             \
+      (const TP *)gamma, (TDX *)dx, (float *)workspace, rows, (int)C)
+#define CS_LN_BWD_MASK(VPL, R)                \
+  if (dx && want_dp) {                        \
+    CS_LN_BWD(VPL, R, true, true);            \
+  } else if (dx) {                            \
+    CS_LN_BWD(VPL, R, true, false);           \
+  } else {                                    \
+    CS_LN_BWD(VPL, R, false, true);           \
+  }
+      if (p.vpl == 2) {
+        CS_LN_BWD_MASK(2, 4)
+      } else if (p.vpl == 4) {
+        CS_LN_BWD_MASK(4, 2)
+      } else {
+        CS_LN_BWD_MASK(8, 1)
+      }
+#undef CS_LN_BWD_MASK
+#undef CS_LN_BWD
+      int st = launch_status();
+      if (st != CS_OK || !want_dp) return st;
+      ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
+          (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, accumulate);
+      return launch_status();
+    }
+  }
+  using U = typename Acc<TX>::type;
+  if (rows > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  if (dx) {
+    ln_bwd_dx_general_kernel<TDY, TX, TDX, TP><<<dim3((unsigned)rows), dim3(kLnThreads), 0, s>>>(
+        (const TDY *)dy, (const TX *)x, (const U *)mean, (const U *)rstd, (const TP *)gamma,
+        (TDX *)dx, C);
+    const int st = launch_status();
+    if (st != CS_OK) return st;
+  }
+  if (want_dp) {
+    ln_bwd_param_general_kernel<TDY, TX, TP>
+        <<<dim3((unsigned)ceil_div(C, (int64_t)64)), dim3(64, 4), 0, s>>>(
+            (const TDY *)dy, (const TX *)x, (const U *)mean, (const U *)rstd, (TP *)dgamma,
+            (TP *)dbeta, rows, C, accumulate);
+    return launch_status();
+  }
+  return CS_OK;
+}
+
+bool wide_ok(int narrow, int other) { return other == narrow || other == CS_F32; }
+
+}  // namespace
+}  // namespace cs_hip
+
+using namespace cs_hip;
+
+extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void *beta, void *y,
+                                    void *mean, void *rstd, int64_t rows, int64_t C, double eps,
+                                    int x_dtype, int y_dtype, int param_dtype, void *stream) {
+  if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
+  if (dtype_size(x_dtype) == 0 || dtype_size(y_dtype) == 0 || dtype_size(param_dtype) == 0)
+    return CS_ERR_UNSUPPORTED;
+  if (!wide_ok(x_dtype, y_dtype) || !wide_ok(x_dtype, param_dtype)) return CS_ERR_UNSUPPORTED;
+  if (x_dtype == CS_F64 && (y_dtype != CS_F64 || param_dtype != CS_F64)) return CS_ERR_UNSUPPORTED;
+  if (rows == 0) return CS_OK;
+  if (!x || !gamma || !y || !mean || !rstd) return CS_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(x, dtype_size(x_dtype)) || !aligned_to(y, dtype_size(y_dtype)) ||
+      !aligned_to(gamma, dtype_size(param_dtype)) ||
+      (beta && !aligned_to(beta, dtype_size(param_dtype))) || !aligned_to(mean, 4) ||
+      !aligned_to(rstd, 4))
+    return CS_ERR_MISALIGNED;
+  const bool aligned =
+      is_aligned16(x) && is_aligned16(y) && is_aligned16(gamma) && (!beta || is_aligned16(beta));
+  hipStream_t s = as_stream(stream);
+#define CS_CALL(TX, TY, TP) \
+  return fwd_typed<TX, TY, TP>(x, gamma, beta, y, mean, rstd, rows, C, eps, aligned, x_dtype, s)
+  const bool y_wide = y_dtype != x_dtype, p_wide = param_dtype != x_dtype;
+  switch (x_dtype) {
+    case CS_F32: CS_CALL(float, float, float);
+    case CS_F64: CS_CALL(double, double, double);
+    case CS_F16:
+      if (y_wide && p_wide) CS_CALL(f16_t, float, float);
+      if (y_wide) CS_CALL(f16_t, float, f16_t);
+      if (p_wide) CS_CALL(f16_t, f16_t, float);
+      CS_CALL(f16_t, f16_t, f16_t);
+    case CS_BF16:
+      if (y_wide && p_wide) CS_CALL(bf16_t, float, float);
+      if (y_wide) CS_CALL(bf16_t, float, bf16_t);
+      if (p_wide) CS_CALL(bf16_t, bf16_t, float);
+      CS_CALL(bf16_t, bf16_t, bf16_t);
+  }
+#undef CS_CALL
+  return CS_ERR_UNSUPPORTED;
+}
+
+extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
+  if (rows <= 0 || C <= 0) return 0;
+  // the fast path's largest grid: the narrowest plan has the fewest rows per
+  // block, so it bounds every dtype
+  FastPlan p;
+  p.vpl = 8;
+  p.rows_per_wave = 1;
+  return (size_t)ln_bwd_blocks(rows, p) * 2 * (size_t)C * sizeof(float);
+}
+
+extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
+                                     const void *rstd, const void *gamma, void *dx, void *dgamma,
+                                     void *dbeta, void *workspace, size_t workspace_bytes,
+                                     int64_t rows, int64_t C, int dy_dtype, int x_dtype,
+                                     int dx_dtype, int param_dtype, int accumulate, void *stream) {
+  if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
+  if (dtype_size(x_dtype) == 0 || dtype_size(dy_dtype) == 0 || dtype_size(dx_dtype) == 0 ||
+      dtype_size(param_dtype) == 0)
+    return CS_ERR_UNSUPPORTED;
+  if (!wide_ok(x_dtype, dy_dtype) || !wide_ok(x_dtype, dx_dtype) || !wide_ok(x_dtype, param_dtype))
+    return CS_ERR_UNSUPPORTED;
+  if (x_dtype == CS_F64 && (dy_dtype != CS_F64 || dx_dtype != CS_F64 || param_dtype != CS_F64))
+    return CS_ERR_UNSUPPORTED;
+  if (!dx && !dgamma && !dbeta) return CS_OK;
+  if (rows == 0) {
+    // an empty batch still defines dgamma/dbeta: zero unless accumulating;
+    // nothing to launch for that without rows, so leave it to the caller
+    return CS_OK;
+  }
+  if (!dy || !x || !mean || !rstd || (dx && !gamma)) return CS_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(dy, dtype_size(dy_dtype)) || !aligned_to(x, dtype_size(x_dtype)) ||
+      (dx && !aligned_to(dx, dtype_size(dx_dtype))) ||
+      (gamma && !aligned_to(gamma, dtype_size(param_dtype))) ||
+      (dgamma && !aligned_to(dgamma, dtype_size(param_dtype))) ||
+      (dbeta && !aligned_to(dbeta, dtype_size(param_dtype))) || !aligned_to(mean, 4) ||
+      !aligned_to(rstd, 4))
+    return CS_ERR_MISALIGNED;
+  const bool aligned = is_aligned16(dy) && is_aligned16(x) && (!dx || is_aligned16(dx)) &&
+                       (!dx || is_aligned16(gamma)) && (!workspace || is_aligned16(workspace));
+  hipStream_t s = as_stream(stream);
+#define CS_CALL(TDY, TX, TDX, TP)                                                              \
+  return bwd_typed<TDY, TX, TDX, TP>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, workspace,   \
+                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, s)
+  const bool dy_wide = dy_dtype != x_dtype, dx_wide = dx_dtype != x_dtype,
+             p_wide = param_dtype != x_dtype;
+  switch (x_dtype) {
+    case CS_F32: CS_CALL(float, float, float, float);
+    case CS_F64: CS_CALL(double, double, double, double);
+    case CS_F16:
+      // autocast runs: fp32 dy and dx with fp32 parameters; plain runs: all f16
+      if (dy_wide && dx_wide && p_wide) CS_CALL(float, f16_t, float, float);
+      if (!dy_wide && !dx_wide && p_wide) CS_CALL(f16_t, f16_t, f16_t, float);
+      if (!dy_wide && !dx_wide && !p_wide) CS_CALL(f16_t, f16_t, f16_t, f16_t);
+      return CS_ERR_UNSUPPORTED;
+    case CS_BF16:
+      if (dy_wide && dx_wide && p_wide) CS_CALL(float, bf16_t, float, float);
+      if (!dy_wide && !dx_wide && p_wide) CS_CALL(bf16_t, bf16_t, bf16_t, float);
+      if (!dy_wide && !dx_wide && !p_wide) CS_CALL(bf16_t, bf16_t, bf16_t, bf16_t);
+      return CS_ERR_UNSUPPORTED;
+  }
+#undef CS_CALL
+  return CS_ERR_UNSUPPORTED;
+}

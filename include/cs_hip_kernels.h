@@ -1,0 +1,251 @@
+/*
+ * C ABI of the gfx950 kernels behind the CoreScheduler op API.
+ *
+ * Every entry point takes plain device pointers, element counts, scalar
+ * hyper-parameters and a HIP stream (passed as void*; NULL is the null
+ * stream).  Entry points enqueue work on that stream and return; none of
+ * them allocates device memory, synchronises the device or the stream, or
+ * touches another stream.  Scratch memory, where a kernel needs it, is a
+ * caller-owned `workspace` whose size the matching *_workspace_bytes call
+ * reports.
+ *
+ * Return value: 0 on success, a negative CS_ERR_* for an argument the
+ * library rejects before launching anything, a positive hipError_t when the
+ * HIP runtime refused a launch.  cs_hip_error_string() names either kind.
+ *
+ * Each declaration cites the reference task body (file:line under the
+ * CoreScheduler tree) whose device work it replaces.  The C++ task bodies
+ * of cs::compute::{CrossEntropy,Embedding,LayerNorm,GeLU} and
+ * cs::optimizer::AdamW are the intended callers; they turn a non-zero
+ * return into CS_ASSERT_TRUE(false, ...).
+ */
+#ifndef CS_HIP_KERNELS_H_
+#define CS_HIP_KERNELS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CS_HIP_ABI_VERSION 1
+
+/* element types */
+enum cs_dtype {
+  CS_F32 = 0,
+  CS_F64 = 1,
+  CS_F16 = 2,
+  CS_BF16 = 3,
+};
+
+/* index types (the reference feeds int64 from its loader and int32 from its
+ * tests: src/data/dataloader.cpp:165, test/test_embedding.cpp:72) */
+enum cs_itype {
+  CS_I32 = 0,
+  CS_I64 = 1,
+};
+
+/* loss reductions; the values are at::Reduction's (None, Mean, Sum) as
+ * stored in CrossEntropy::State::Args::reduction
+ * (include/compute/cross_entropy.h:38-42) */
+enum cs_reduction {
+  CS_REDUCTION_NONE = 0,
+  CS_REDUCTION_MEAN = 1,
+  CS_REDUCTION_SUM = 2,
+};
+
+/* GeLU flavours: at::gelu's `approximate` argument ("none" / "tanh") */
+enum cs_gelu_mode {
+  CS_GELU_ERF = 0,
+  CS_GELU_TANH = 1,
+};
+
+enum cs_error {
+  CS_OK = 0,
+  CS_ERR_INVALID_ARGUMENT = -1, /* null pointer, negative size, bad enum   */
+  CS_ERR_UNSUPPORTED = -2,      /* dtype combination that has no kernel     */
+  CS_ERR_MISALIGNED = -3,       /* pointer not aligned to its element size  */
+  CS_ERR_WORKSPACE = -4,        /* workspace missing or too small           */
+  CS_ERR_TOO_LARGE = -5,        /* size beyond what the launch can address  */
+};
+
+int cs_hip_abi_version(void);
+const char *cs_hip_error_string(int code);
+
+/* ------------------------------------------------------------------------
+ * AdamW
+ * replaces stepKernel / stepKernelAmsgrad and the step<UpT,T> kernels,
+ * src/optimizer/adamw.cu:35-60, :62-90, :93-151.
+ *
+ * All of w, dw, m, v (and v_max) hold `n` elements of `dtype`; arithmetic is
+ * in float (double for CS_F64) in the reference's operation order.  The bias
+ * corrections 1/(1-beta^t) are formed on the host in double and narrowed, as
+ * adamw.cu:116-117 does.  v_max == NULL selects the plain step, non-NULL the
+ * amsgrad step.  `t` is the step count AFTER the increment the caller makes
+ * at submit time (src/optimizer/adamw.cpp:112), so the first step has t == 1.
+ * ---------------------------------------------------------------------- */
+int cs_adamw_step(void *w, const void *dw, void *m, void *v, void *v_max,
+                  int64_t n, int dtype, double lr, double beta1, double beta2,
+                  double eps, double weight_decay, int64_t t, void *stream);
+
+/* One launch for a whole parameter set (the 148 launches per step of
+ * src/module/adamw.cpp:32-38 become one).  The caller fills an array of
+ * descriptors, asks the library to lay out a device table for them in HOST
+ * memory, copies those bytes to the device itself (any way it likes) and
+ * passes the device copy to the step.  Pointers in the table may be
+ * refreshed and re-uploaded every step (gradients are re-allocated after
+ * zero_grad in the reference: src/compute/embedding.cpp:54). */
+typedef struct cs_adamw_tensor {
+  void *w;
+  const void *dw;
+  void *m;
+  void *v;
+  void *v_max; /* NULL unless amsgrad */
+  int64_t n;
+} cs_adamw_tensor;
+
+size_t cs_adamw_multi_table_bytes(int64_t n_tensors);
+/* Writes the table for `tensors` into host_table (table_bytes long) and the
+ * number of workgroup slots the launch needs into *n_slots.  The layout
+ * depends on `dtype`; pass the same dtype to cs_adamw_multi_step. */
+int cs_adamw_multi_build_table(const cs_adamw_tensor *tensors,
+                               int64_t n_tensors, int dtype, void *host_table,
+                               size_t table_bytes, int64_t *n_slots);
+int cs_adamw_multi_step(const void *device_table, int64_t n_tensors,
+                        int64_t n_slots, int dtype, int amsgrad, double lr,
+                        double beta1, double beta2, double eps,
+                        double weight_decay, int64_t t, void *stream);
+
+/* ------------------------------------------------------------------------
+ * GeLU
+ * replaces at::gelu / at::gelu_backward in the task bodies of
+ * src/compute/gelu.cpp:39 and :61-62 (erf form; the reference never passes
+ * `approximate`).  CS_GELU_TANH is at::gelu(x, "tanh").  x, y, dy, dx hold
+ * `n` elements of `dtype`; the arithmetic is fp32 for f16/bf16 storage.
+ * ---------------------------------------------------------------------- */
+int cs_gelu_forward(const void *x, void *y, int64_t n, int dtype, int mode,
+                    void *stream);
+int cs_gelu_backward(const void *dy, const void *x, void *dx, int64_t n,
+                     int dtype, int mode, void *stream);
+
+/* ------------------------------------------------------------------------
+ * LayerNorm over the last dimension
+ * forward replaces at::native_layer_norm, src/compute/layer_norm.cpp:163-169
+ * and :198-204; backward replaces both at::native_layer_norm_backward calls,
+ * :263-266 (dx) and :321-334 / :375-383 (dgamma, dbeta, with += when the
+ * gradient already exists).
+ *
+ * x, y: [rows, C] row-major contiguous.  gamma, beta: [C] (beta may be NULL:
+ * the reference's bias=false path).  mean, rstd: [rows] fp32 (fp64 when
+ * x_dtype is CS_F64), rstd = 1/sqrt(biased variance + eps).
+ * x_dtype: storage of x.  y_dtype: storage of y, either x_dtype or CS_F32
+ * (what autocast produces for bf16 x).  param_dtype: storage of gamma/beta,
+ * either x_dtype or CS_F32.
+ * ---------------------------------------------------------------------- */
+int cs_layernorm_forward(const void *x, const void *gamma, const void *beta,
+                         void *y, void *mean, void *rstd, int64_t rows,
+                         int64_t C, double eps, int x_dtype, int y_dtype,
+                         int param_dtype, void *stream);
+
+size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C);
+/* Any of dx, dgamma, dbeta may be NULL (the reference's output masks
+ * {1,0,0}, {0,1,1}, {0,1,0}); dgamma/dbeta are stored in param_dtype and,
+ * when accumulate != 0, added to what is already there.  dy is stored as
+ * dy_dtype (x_dtype or CS_F32), dx as dx_dtype (same choice).  workspace
+ * is needed whenever dgamma or dbeta is requested. */
+int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
+                          const void *rstd, const void *gamma, void *dx,
+                          void *dgamma, void *dbeta, void *workspace,
+                          size_t workspace_bytes, int64_t rows, int64_t C,
+                          int dy_dtype, int x_dtype, int dx_dtype,
+                          int param_dtype, int accumulate, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Embedding
+ * forward replaces torch::embedding, src/compute/embedding.cpp:117-121:
+ * out[i, :] = weight[indices[i], :], a byte-exact copy.  An index outside
+ * [0, num_weights) yields a zero row and never reads out of bounds.
+ * ---------------------------------------------------------------------- */
+int cs_embedding_forward(const void *weight, const void *indices, void *out,
+                         int64_t n_indices, int64_t C, int64_t num_weights,
+                         int dtype, int idx_dtype, void *stream);
+
+/* Token + position embedding in one pass: out[b,t,:] = wte[ids[b,t],:] +
+ * wpe[t,:], replacing the two gathers, broadcast_to and add of
+ * example/gpt2/gpt2_single_device.cpp:541-545.  The sum is formed in fp32
+ * and rounded once, which for f16/bf16 equals the reference's add bit for
+ * bit. */
+int cs_embedding_forward_add(const void *wte, const void *wpe,
+                             const void *indices, void *out, int64_t B,
+                             int64_t T, int64_t C, int64_t num_weights,
+                             int dtype, int idx_dtype, void *stream);
+
+/* backward replaces at::embedding_backward (+ the += of an existing
+ * gradient), src/compute/embedding.cpp:147-157: dense dweight[num_weights,C],
+ * dweight[k] = sum over {i : indices[i]==k, k != padding_idx} of dout[i],
+ * rows never indexed are zero (left untouched when accumulate != 0).
+ * Sums are formed in fp32 (fp64 for CS_F64) in ascending order of i, by
+ * sorting (index, i) pairs and reducing segments, so results do not depend
+ * on scheduling.  padding_idx < 0 means none. */
+size_t cs_embedding_backward_workspace_bytes(int64_t n_indices, int64_t C,
+                                             int64_t num_weights);
+int cs_embedding_backward(const void *dout, const void *indices,
+                          void *dweight, void *workspace,
+                          size_t workspace_bytes, int64_t n_indices, int64_t C,
+                          int64_t num_weights, int64_t padding_idx, int dtype,
+                          int idx_dtype, int accumulate, void *stream);
+
+/* Token and position table gradients of out[b,t,:] = wte[ids[b,t],:] +
+ * wpe[t,:] from one dout[B,T,C]: dwte as cs_embedding_backward (no padding
+ * index), dwpe[t,:] (+)= sum_b dout[b,t,:] in ascending b.  Replaces
+ * Utils::sum(dx,0), wpe->backward and wte->backward of
+ * example/gpt2/gpt2_single_device.cpp:565-567 with one call.  Workspace as
+ * cs_embedding_backward_workspace_bytes(B*T, C, num_weights). */
+int cs_embedding_backward_fused(const void *dout, const void *indices,
+                                void *dwte, void *dwpe, void *workspace,
+                                size_t workspace_bytes, int64_t B, int64_t T,
+                                int64_t C, int64_t num_weights, int dtype,
+                                int idx_dtype, int accumulate, void *stream);
+
+/* Position-table gradient: dwpe[t,:] (+)= sum_b dout[b,t,:], replacing
+ * Utils::sum(dx, 0) followed by wpe->backward with arange positions,
+ * example/gpt2/gpt2_single_device.cpp:565-566. */
+int cs_embedding_backward_positions(const void *dout, void *dwpe, int64_t B,
+                                    int64_t T, int64_t C, int dtype,
+                                    int accumulate, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Fused classifier: row softmax + cross-entropy loss + dlogits
+ * replaces at::log_softmax + at::nll_loss_forward
+ * (src/compute/cross_entropy.cpp:57-63) and at::nll_loss_backward +
+ * at::_log_softmax_backward_data (:103-109) with one pass over the logits.
+ *
+ * logits: [N, row_stride] row-major, columns [0, V) are classes, columns
+ * [V, row_stride) are padding that is ignored on input.
+ * targets: [N] int64; rows whose target equals ignore_index contribute no
+ * loss and get zero dlogits.
+ * row_loss: [N] fp32, written for every reduction (NULL: not wanted unless
+ * reduction is NONE).  loss: one fp32 (MEAN or SUM; ignored for NONE).
+ * total_weight: one fp32 = number of rows not ignored (may be NULL).
+ * dlogits: [N, row_stride] of dlogits_dtype (logits' dtype or CS_F32), may
+ * alias logits when the dtypes match (in-place), may be NULL (loss only).
+ * dlogits = (softmax(logits) - onehot(target)) * s, s = dloss / total_weight
+ * for MEAN and dloss otherwise; padding columns are written as zero.  The
+ * reference has no upstream gradient (it passes ones_like(loss)):
+ * dloss = 1 reproduces it.
+ * ---------------------------------------------------------------------- */
+size_t cs_fused_classifier_workspace_bytes(int64_t N);
+int cs_fused_classifier(const void *logits, void *dlogits,
+                        const int64_t *targets, float *row_loss, float *loss,
+                        float *total_weight, void *workspace,
+                        size_t workspace_bytes, int64_t N, int64_t V,
+                        int64_t row_stride, int64_t ignore_index,
+                        int reduction, float dloss, int dtype,
+                        int dlogits_dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CS_HIP_KERNELS_H_ */

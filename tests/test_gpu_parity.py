@@ -1,0 +1,471 @@
+"""Parity of the gfx950 kernels with the CPU oracle, through the C ABI.
+
+Every test feeds the same seeded inputs to the HIP path (core_scheduler_amd.ops
+-> ctypes -> libcs_hip_kernels.so) and to the oracle (oracle/cs_oracle.c).
+The bar (see tests/_util.py): bit-exact for the gather and gather-add;
+fp32 within rtol 1e-5 plus the atol stated at each call; 16-bit outputs within
+1 ulp of the oracle's once-rounded value.
+Shapes follow the reference's own tests (test/test_*.cpp) and the benchmark
+configurations; the largest ones are checked through the oracle on a sample of
+rows plus properties that hold at any size.
+"""
+import math
+
+import pytest
+import torch
+
+from _util import (assert_bit_exact, assert_close, gpt2_param_shapes, randint, randn, zipf_ids)
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from core_scheduler_amd import ops as _ops
+
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def co():
+    from oracle import c_oracle
+
+    return c_oracle
+
+
+def dev(t):
+    return None if t is None else t.to(DEV)
+
+
+HYPER = dict(lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+
+
+# ------------------------------------------------------------------ AdamW
+@pytest.mark.parametrize("n", [1, 127, 4096, 4097, 100003])
+@pytest.mark.parametrize("amsgrad", [False, True])
+def test_adamw_flat_f32(ops, co, n, amsgrad):
+    w = randn(n, 1, std=0.02)
+    m, v = torch.zeros(n), torch.zeros(n)
+    x = torch.zeros(n) if amsgrad else None
+    gw, gm, gv, gx = dev(w), dev(m), dev(v), dev(x)
+    for t in range(1, 4):
+        g = randn(n, 10 + t, std=1e-3)
+        ops.adamw_step(gw, dev(g), gm, gv, t=t, v_max=gx, **HYPER)
+        w, m, v, x = co.adamw_step(w, g, m, v, t=t, v_max=x, **HYPER)
+    assert_close(gw, w, atol=1e-8, name="w")
+    assert_close(gm, m, atol=1e-10, name="m")
+    assert_close(gv, v, atol=1e-13, name="v")
+    if amsgrad:
+        assert_close(gx, x, atol=1e-13, name="v_max")
+
+
+def test_adamw_reference_test_case(ops):
+    # test/test_adamw.cpp:63-103, closed form written out there, its own tolerances
+    for size in (128, 512, 1024):
+        x = torch.rand(size, generator=torch.Generator().manual_seed(1))
+        dx = torch.rand(size, generator=torch.Generator().manual_seed(2))
+        gw, gm, gv = dev(x), dev(torch.zeros(size)), dev(torch.zeros(size))
+        ops.adamw_step(gw, dev(dx), gm, gv, lr=1.0, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-2, t=1)
+        xt = x - 1.0 * 1e-2 * x
+        mt = (1 - 0.9) * dx
+        vt = (1 - 0.999) * dx.square()
+        xt = xt - 1.0 * (mt / (1 - 0.9)) / ((vt / (1 - 0.999)).sqrt() + 1e-8)
+        assert torch.allclose(gw.cpu(), xt, 1e-4, 1e-5)
+        assert torch.allclose(gm.cpu(), mt, 1e-4, 1e-5)
+        assert torch.allclose(gv.cpu(), vt, 1e-4, 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.bfloat16, torch.float16])
+def test_adamw_other_dtypes(ops, co, dtype):
+    n = 9001
+    w, g = randn(n, 2, std=0.5, dtype=dtype), randn(n, 3, std=0.1, dtype=dtype)
+    m, v = torch.zeros(n, dtype=dtype), torch.zeros(n, dtype=dtype)
+    gw, gm, gv = dev(w), dev(m), dev(v)
+    ops.adamw_step(gw, dev(g), gm, gv, t=1, **HYPER)
+    w2, m2, v2, _ = co.adamw_step(w, g, m, v, t=1, **HYPER)
+    atol = 1e-14 if dtype == torch.float64 else 1e-7
+    assert_close(gw, w2, atol=atol, name="w")
+    assert_close(gm, m2, atol=atol, name="m")
+    assert_close(gv, v2, atol=atol * 1e-3, name="v")
+
+
+def test_adamw_unaligned_views(ops, co):
+    # element 1 of an aligned buffer: 4-byte but not 16-byte aligned -> scalar path
+    n = 5000
+    bufs = [randn(n + 1, s, std=0.02) for s in (4, 5)] + [torch.zeros(n + 1), torch.zeros(n + 1)]
+    gb = [dev(b) for b in bufs]
+    ops.adamw_step(gb[0][1:], gb[1][1:], gb[2][1:], gb[3][1:], t=1, **HYPER)
+    w2, m2, v2, _ = co.adamw_step(bufs[0][1:], bufs[1][1:], bufs[2][1:], bufs[3][1:], t=1, **HYPER)
+    assert_close(gb[0][1:], w2, atol=1e-8, name="w")
+    assert gb[0][0].item() == bufs[0][0].item() and gb[2][0].item() == 0  # the neighbour is untouched
+
+
+def test_adamw_multi_tensor_small_set(ops, co):
+    shapes = [(7,), (4096,), (33, 129), (4097,), (1,), (3, 5, 7)]
+    ws = [randn(s, 20 + i, std=0.02) for i, s in enumerate(shapes)]
+    gs = [randn(s, 40 + i, std=1e-3) for i, s in enumerate(shapes)]
+    gws, ggs = [dev(w) for w in ws], [dev(g) for g in gs]
+    flat = [w.clone() for w in gws]
+    opt = ops.MultiTensorAdamW(gws, ggs, t=0, **HYPER)
+    fm = [torch.zeros_like(w) for w in flat]
+    fv = [torch.zeros_like(w) for w in flat]
+    for t in range(1, 4):
+        opt.step()
+        for w, g, m, v in zip(flat, ggs, fm, fv):
+            ops.adamw_step(w, g, m, v, t=t, **HYPER)
+    ms = [torch.zeros(s) for s in shapes]
+    vs = [torch.zeros(s) for s in shapes]
+    for i in range(len(shapes)):
+        w, m, v = ws[i], ms[i], vs[i]
+        for t in range(1, 4):
+            w, m, v, _ = co.adamw_step(w, gs[i], m, v, t=t, **HYPER)
+        assert_close(gws[i], w.reshape(shapes[i]), atol=1e-8, name=f"w[{i}]")
+        assert_close(opt.m[i], m.reshape(shapes[i]), atol=1e-10, name=f"m[{i}]")
+        assert_bit_exact(gws[i], flat[i], f"multi == flat [{i}]")  # same arithmetic, two launch shapes
+
+
+def test_adamw_gpt2_small_ten_steps(ops, co):
+    """Benchmark configuration 0: all 148 GPT-2-small tensors, 10 steps, fresh grads each step."""
+    shapes = gpt2_param_shapes()
+    sizes = [math.prod(s) for s in shapes]
+    total = sum(sizes)
+    assert len(shapes) == 148 and total == 124_439_808
+    w = randn(total, 1337, std=0.02)
+    gw_flat = dev(w)
+    gg_flat = torch.empty(total, device=DEV)
+    offs = [0]
+    for s in sizes:
+        offs.append(offs[-1] + s)
+    gws = [gw_flat[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+    ggs = [gg_flat[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+    opt = ops.MultiTensorAdamW(gws, ggs, t=0, **HYPER)
+    m, v = torch.zeros(total), torch.zeros(total)
+    for t in range(1, 11):
+        g = randn(total, 2000 + t, std=1e-3)
+        gg_flat.copy_(g)
+        opt.step()
+        w, m, v, _ = co.adamw_step(w, g, m, v, t=t, **HYPER)
+    assert_close(gw_flat, w, atol=1e-8, name="w after 10 steps")
+    assert_close(torch.cat([x.flatten() for x in opt.m]), m, atol=1e-10, name="m")
+    assert_close(torch.cat([x.flatten() for x in opt.v]), v, atol=1e-13, name="v")
+
+
+# ------------------------------------------------------------------- GeLU
+GELU_ATOL = {torch.float32: 1e-6, torch.float64: 1e-14, torch.bfloat16: 1e-6, torch.float16: 1e-6}
+
+
+@pytest.mark.parametrize("mode", ["none", "tanh"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+@pytest.mark.parametrize("n", [1, 1000, 8192, 2 * 1024 * 768 + 3])
+def test_gelu(ops, co, mode, dtype, n):
+    # reference shapes: B=2, T in {128,512,1024} (test/test_gelu.cpp:59-102)
+    x = randn(n, 3, std=1.5, dtype=dtype)
+    dy = randn(n, 4, dtype=dtype)
+    atol = GELU_ATOL[dtype]
+    assert_close(ops.gelu_forward(dev(x), mode), co.gelu_forward(x, mode), atol=atol, name="fwd")
+    # backward: the fp32 floor scales with |dy| (up to ~5) and |x|
+    assert_close(ops.gelu_backward(dev(dy), dev(x), mode), co.gelu_backward(dy, x, mode), atol=atol * 5, name="bwd")
+
+
+def test_gelu_edge_values(ops, co):
+    x = torch.tensor([0.0, -0.0, 1e-30, -1e-30, 20.0, -20.0, 88.0, -88.0, float("inf"), float("-inf")] * 8)
+    for mode in ("none", "tanh"):
+        for dtype in (torch.float32, torch.bfloat16):
+            xx = x.to(dtype)
+            got = ops.gelu_forward(dev(xx), mode).cpu().float()
+            want = co.gelu_forward(xx, mode).float()
+            finite = torch.isfinite(x)
+            assert_close(got[finite], want[finite], atol=1e-6, name=f"{mode} {dtype}")
+            assert got[8] == float("inf")  # gelu(+inf) = +inf; gelu(-inf) is 0 * inf in ATen's form (NaN)
+
+
+def test_gelu_config3_full_size(ops, co):
+    x = randn((8192, 3072), 1340, std=1.5, dtype=torch.bfloat16)
+    dy = randn((8192, 3072), 1341, dtype=torch.bfloat16)
+    assert_close(ops.gelu_forward(dev(x), "tanh"), co.gelu_forward(x, "tanh"), atol=1e-6, name="fwd")
+    assert_close(ops.gelu_backward(dev(dy), dev(x), "tanh"), co.gelu_backward(dy, x, "tanh"), atol=5e-6, name="bwd")
+
+
+# -------------------------------------------------------------- LayerNorm
+def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
+    x = randn((rows, C), 50, dtype=x_dtype)
+    gamma = randn(C, 51, std=0.02, mean=1.0, dtype=p_dtype)
+    beta = randn(C, 52, std=0.02, dtype=p_dtype) if bias else None
+    dy = randn((rows, C), 53, dtype=x_dtype)
+    y, mean, rstd = ops.layernorm_forward(dev(x), dev(gamma), dev(beta), 1e-5)
+    y2, mean2, rstd2 = co.layernorm_forward(x, gamma, beta, 1e-5)
+    wide = x_dtype != torch.float64
+    assert mean.dtype == (torch.float32 if wide else torch.float64)
+    assert_close(y, y2, atol=atol_y, name="y")
+    assert_close(mean, mean2, atol=1e-7, name="mean")
+    assert_close(rstd, rstd2, atol=1e-6, name="rstd")
+    # backward from the oracle's statistics, so only the backward kernel is judged
+    dx, dg, db = ops.layernorm_backward(dev(dy), dev(x), dev(mean2), dev(rstd2), dev(gamma), need_dbeta=bias)
+    dx2, dg2, db2 = co.layernorm_backward(dy, x, mean2, rstd2, gamma)
+    assert_close(dx, dx2, atol=5e-6, name="dx")
+    # column sums over `rows` terms of O(1): fp32 accumulation error grows like sqrt(rows) * 1e-7
+    atol_p = 1e-14 if not wide else 2e-7 * math.sqrt(rows) + 1e-6
+    if p_dtype in (torch.bfloat16, torch.float16):
+        atol_p = 1e-6
+    assert_close(dg, dg2, atol=atol_p, name="dgamma")
+    if bias:
+        assert_close(db, db2, atol=atol_p, name="dbeta")
+    else:
+        assert db is None
+
+
+@pytest.mark.parametrize("rows,C,x_dtype,p_dtype", [
+    (8192, 768, torch.bfloat16, torch.float32),     # benchmark configuration 3
+    (2048, 1600, torch.bfloat16, torch.float32),    # XL width (2 rows per wave plan)
+    (1024, 384, torch.float32, torch.float32),      # test/test_layer_norm.cpp:63-96 width
+    (513, 768, torch.float16, torch.float16),
+    (300, 768, torch.bfloat16, torch.bfloat16),
+    (77, 4096, torch.bfloat16, torch.float32),      # 8 vectors per lane plan
+    (5, 768, torch.float32, torch.float32),         # fewer rows than one workgroup
+    (64, 50, torch.float32, torch.float32),         # C not a multiple of the vector width
+    (33, 10000, torch.bfloat16, torch.float32),     # beyond the register plans
+    (128, 384, torch.float64, torch.float64),       # test/test_layer_norm.cpp:99-134
+])
+def test_layernorm(ops, co, rows, C, x_dtype, p_dtype):
+    _ln_case(ops, co, rows, C, x_dtype, p_dtype)
+
+
+def test_layernorm_without_bias(ops, co):
+    _ln_case(ops, co, 256, 768, torch.bfloat16, torch.float32, bias=False)
+    _ln_case(ops, co, 64, 50, torch.float32, torch.float32, bias=False)
+
+
+def test_layernorm_reference_test_values(ops):
+    # test/test_layer_norm.cpp:63-96: x = rand, weight 1, bias 0, against torch's LayerNorm (ATen CPU here)
+    x = torch.rand((16, 256, 384), generator=torch.Generator().manual_seed(1))
+    w, b = torch.ones(384), torch.zeros(384)
+    y, mean, rstd = ops.layernorm_forward(dev(x), dev(w), dev(b), 1e-5)
+    xr = x.clone().requires_grad_()
+    ln = torch.nn.LayerNorm(384)
+    yr = ln(xr)
+    dy = torch.rand(yr.shape, generator=torch.Generator().manual_seed(2))
+    yr.backward(dy)
+    dx, dg, db = ops.layernorm_backward(dev(dy), dev(x), mean, rstd, dev(w))
+    assert_close(y, yr.detach(), atol=2e-6, name="y")
+    assert_close(dx, xr.grad, atol=5e-6, name="dx")
+    assert_close(dg, ln.weight.grad, atol=1e-3, rtol=1e-5, name="dgamma")  # sums of 4096 terms ~ 2e3
+    assert_close(db, ln.bias.grad, atol=1e-3, rtol=1e-5, name="dbeta")
+
+
+def test_layernorm_autocast_dtypes(ops, co):
+    # test/test_autocast.cpp:112-156: bf16 x, fp32 parameters, fp32 y and fp32 dy/dx
+    rows, C = 512, 768
+    x = randn((rows, C), 60, dtype=torch.bfloat16)
+    gamma, beta = randn(C, 61, std=0.02, mean=1.0), randn(C, 62, std=0.02)
+    dy = randn((rows, C), 63)
+    y, mean, rstd = ops.layernorm_forward(dev(x), dev(gamma), dev(beta), 1e-5, out_dtype=torch.float32)
+    y2, mean2, rstd2 = co.layernorm_forward(x, gamma, beta, 1e-5, out_dtype=torch.float32)
+    assert y.dtype == torch.float32
+    assert_close(y, y2, atol=2e-6, name="y fp32")
+    dx, dg, db = ops.layernorm_backward(dev(dy), dev(x), mean, rstd, dev(gamma), dx_dtype=torch.float32)
+    dx2, dg2, db2 = co.layernorm_backward(dy, x, mean2, rstd2, gamma, out_dtype=torch.float32)
+    assert_close(dx, dx2, atol=5e-6, name="dx fp32")
+    assert_close(dg, dg2, atol=1e-5, name="dgamma")
+    assert_close(db, db2, atol=1e-5, name="dbeta")
+
+
+def test_layernorm_masks_and_accumulate(ops, co):
+    rows, C = 700, 768
+    x = randn((rows, C), 70, dtype=torch.bfloat16)
+    gamma = randn(C, 71, std=0.02, mean=1.0)
+    dy = randn((rows, C), 72, dtype=torch.bfloat16)
+    _, mean, rstd = co.layernorm_forward(x, gamma, None, 1e-5)
+    gx, gdy, gm, gr, gg = dev(x), dev(dy), dev(mean), dev(rstd), dev(gamma)
+    full = ops.layernorm_backward(gdy, gx, gm, gr, gg)
+    only_dx = ops.layernorm_backward(gdy, gx, gm, gr, gg, need_dgamma=False, need_dbeta=False)
+    only_p = ops.layernorm_backward(gdy, gx, gm, gr, gg, need_dx=False)
+    assert only_dx[1] is None and only_dx[2] is None and only_p[0] is None
+    assert_bit_exact(only_dx[0], full[0], "dx alone")          # the reference's mask {1,0,0}
+    assert_bit_exact(only_p[1], full[1], "dgamma alone")       # mask {0,1,1}
+    assert_bit_exact(only_p[2], full[2], "dbeta alone")
+    # += into existing gradients (src/compute/layer_norm.cpp:325-334)
+    dg0, db0 = randn(C, 73), randn(C, 74)
+    gdg, gdb = dev(dg0), dev(db0)
+    ops.layernorm_backward(gdy, gx, gm, gr, gg, need_dx=False, dgamma=gdg, dbeta=gdb)
+    _, dg2, db2 = co.layernorm_backward(dy, x, mean, rstd, gamma, dgamma=dg0, dbeta=db0)
+    assert_close(gdg, dg2, atol=1e-5, name="dgamma +=")
+    assert_close(gdb, db2, atol=1e-5, name="dbeta +=")
+    # determinism: same bits on a second run
+    again = ops.layernorm_backward(gdy, gx, gm, gr, gg)
+    for a, b in zip(again, full):
+        assert_bit_exact(a, b, "rerun")
+
+
+# -------------------------------------------------------------- Embedding
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+@pytest.mark.parametrize("idx_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("V,C,B,T", [(4095, 512, 2, 1024), (97, 24, 3, 11), (50, 7, 2, 5)])
+def test_embedding_forward_bit_exact(ops, co, dtype, idx_dtype, V, C, B, T):
+    w = randn((V, C), 80, dtype=dtype)
+    wpe = randn((T, C), 81, dtype=dtype)
+    ids = randint(0, V, (B, T), 82, dtype=idx_dtype)
+    assert_bit_exact(ops.embedding_forward(dev(w), dev(ids)), co.embedding_forward(w, ids), "gather")
+    assert_bit_exact(ops.embedding_forward_add(dev(w), dev(wpe), dev(ids)), co.embedding_forward_add(w, wpe, ids),
+                     "gather-add")
+
+
+def test_embedding_forward_out_of_range_ids_give_zero_rows(ops):
+    w = randn((10, 16), 83)
+    ids = torch.tensor([[0, 9, 10, -1, 3]], dtype=torch.int64)
+    out = ops.embedding_forward(dev(w), dev(ids)).cpu()
+    assert torch.equal(out[0, 0], w[0]) and torch.equal(out[0, 1], w[9]) and torch.equal(out[0, 4], w[3])
+    assert (out[0, 2] == 0).all() and (out[0, 3] == 0).all()
+
+
+EMB_ATOL = {torch.float32: 2e-5, torch.float16: 1e-6, torch.bfloat16: 1e-6, torch.float64: 1e-12}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_embedding_backward_reference_test_case(ops, co, dtype):
+    # test/test_embedding.cpp:58-97: B 2, T 1024, vocab 4095, d 512, int32 ids in [0, 3): 2048 rows onto 3
+    B, T, V, C = 2, 1024, 4095, 512
+    ids = randint(0, 3, (B, T), 90, dtype=torch.int32)
+    dout = randn((B, T, C), 91, dtype=dtype)
+    got = ops.embedding_backward(dev(dout), dev(ids), V)
+    # sums of ~680 N(0,1) terms are ~26 in size: fp32 accumulation leaves ~1e-5 absolute
+    assert_close(got, co.embedding_backward(dout, ids, V), atol=EMB_ATOL[dtype], name="dweight")
+    assert (got[3:] == 0).all()
+    assert_bit_exact(ops.embedding_backward(dev(dout), dev(ids), V), got, "rerun is bitwise identical")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("n,V,C", [(1, 5, 8), (8, 5, 8), (9, 40, 16), (2048, 300, 64), (2049, 1000, 72),
+                                   (5000, 7, 128), (4097, 100000, 8), (300, 50, 12), (64, 20, 7)])
+def test_embedding_backward_shapes(ops, co, dtype, n, V, C):
+    ids = randint(0, V, (n,), 92)
+    dout = randn((n, C), 93, dtype=dtype)
+    got = ops.embedding_backward(dev(dout), dev(ids), V)
+    assert_close(got, co.embedding_backward(dout, ids, V), atol=EMB_ATOL[dtype] * 4, name="dweight")
+
+
+def test_embedding_backward_padding_accumulate_and_bad_ids(ops, co):
+    n, V, C = 3000, 64, 32
+    ids = randint(0, V, (n,), 94)
+    dout = randn((n, C), 95)
+    got = ops.embedding_backward(dev(dout), dev(ids), V, padding_idx=5)
+    assert (got[5] == 0).all()
+    assert_close(got, co.embedding_backward(dout, ids, V, padding_idx=5), atol=2e-5, name="padding_idx")
+    base = randn((V, C), 96)
+    acc = dev(base)
+    ops.embedding_backward(dev(dout), dev(ids), V, dweight=acc)
+    assert_close(acc, co.embedding_backward(dout, ids, V, dweight=base), atol=2e-5, name="+=")
+    bad = ids.clone()
+    bad[::7] = V + 3
+    bad[1::7] = -2
+    assert_close(ops.embedding_backward(dev(dout), dev(bad), V), co.embedding_backward(dout, bad, V), atol=2e-5,
+                 name="out-of-range ids are skipped")
+
+
+@pytest.mark.parametrize("kind", ["uniform", "zipf"])
+def test_embedding_config1(ops, co, kind):
+    """Benchmark configuration 1: wte 50257x768, wpe 1024x768 bf16, B 8, T 1024."""
+    V, C, B, T = 50257, 768, 8, 1024
+    wte, wpe = randn((V, C), 1338, std=0.02, dtype=torch.bfloat16), randn((T, C), 1339, std=0.02, dtype=torch.bfloat16)
+    ids = (randint(0, V, (B * T,), 100) if kind == "uniform" else zipf_ids(B * T, V, 101)).reshape(B, T)
+    dout = randn((B, T, C), 102, dtype=torch.bfloat16)
+    assert_bit_exact(ops.embedding_forward_add(dev(wte), dev(wpe), dev(ids)), co.embedding_forward_add(wte, wpe, ids),
+                     "gather-add")
+    dwte, dwpe = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_close(dwte, co.embedding_backward(dout, ids, V), atol=1e-6, name="dwte")
+    assert_close(dwpe, co.embedding_backward_positions(dout), atol=1e-6, name="dwpe")
+    again = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_bit_exact(again[0], dwte, "dwte rerun")
+    # accumulate into existing gradients
+    ops.embedding_backward_fused(dev(dout), dev(ids), V, dwte=again[0], dwpe=again[1])
+    assert_close(again[1], co.embedding_backward_positions(dout, dwpe=dwpe.cpu()), atol=1e-6, name="dwpe +=")
+    assert_close(again[0], co.embedding_backward(dout, ids, V, dweight=dwte.cpu()), atol=1e-6, name="dwte +=")
+    assert_close(ops.embedding_backward_positions(dev(dout)), co.embedding_backward_positions(dout), atol=1e-6,
+                 name="positions alone")
+
+
+# ---------------------------------------------------------- Cross entropy
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_cross_entropy_reference_test_case(ops, co, reduction, dtype):
+    # test/test_cross_entropy.cpp:69-99: x = rand [B*256, 384], targets randint [0,384); fewer rows here
+    N, V = 4096, 384
+    x = torch.rand((N, V), generator=torch.Generator().manual_seed(1)).to(dtype)
+    t = randint(0, V, (N,), 110)
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t), reduction=reduction)
+    loss2, row2, d2, tw2 = co.cross_entropy(x, t, reduction=reduction)
+    assert_close(loss.double(), loss2.double(), atol=1e-5 if reduction != "sum" else 1e-1, name="loss")
+    assert_close(row.double(), row2.double(), atol=2e-6, name="row loss")
+    assert_close(d, d2, atol=1e-9 if reduction == "mean" else 1e-7, name="dlogits")
+    assert tw.item() == tw2.item() == N
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("N,V,stride", [(64, 50257, 50304), (8, 50304, 50304), (33, 1000, 1024), (16, 4000, 4096),
+                                        (5, 16385, 16392), (7, 100, 100), (3, 130000, 130048), (4, 77, 77)])
+def test_cross_entropy_shapes(ops, co, dtype, N, V, stride):
+    x = randn((N, stride), 111, std=2.0, dtype=dtype)
+    t = randint(0, V, (N,), 112)
+    if N > 4:
+        t[1] = -100  # an ignored row
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t), V)
+    loss2, row2, d2, tw2 = co.cross_entropy(x, t, V)
+    assert_close(loss, loss2.float(), atol=1e-5, name="loss")
+    assert_close(row, row2.float(), atol=1e-5, name="row loss")
+    # softmax entries are ~1/V/N: a relative bar with a floor far below them
+    assert_close(d, d2, atol=1e-10, name="dlogits")
+    assert (d[:, V:] == 0).all()
+    assert tw.item() == tw2.item()
+
+
+def test_cross_entropy_inplace_amp_and_dloss(ops, co):
+    N, V, stride = 48, 50257, 50304
+    x = randn((N, stride), 113, std=2.0, dtype=torch.bfloat16)
+    t = randint(0, V, (N,), 114)
+    _, _, d2, _ = co.cross_entropy(x, t, V)
+    gx = dev(x)
+    loss, row, d, _ = ops.fused_classifier(gx, dev(t), V, inplace=True)
+    assert d.data_ptr() == gx.data_ptr()
+    assert_close(gx, d2, atol=1e-10, name="in-place dlogits")
+    # fp32 gradient from bf16 logits (the autocast rule, test/test_cross_entropy.cpp:102-139)
+    _, _, d32, _ = ops.fused_classifier(dev(x), dev(t), V, dlogits_dtype=torch.float32)
+    _, _, d32o, _ = co.cross_entropy(x, t, V, dlogits_dtype=torch.float32)
+    assert_close(d32, d32o, atol=1e-10, name="fp32 dlogits")
+    # upstream gradient, negative too; loss only
+    for dloss in (0.25, -3.0, 0.0):
+        _, _, dd, _ = ops.fused_classifier(dev(x), dev(t), V, dloss=dloss, dlogits_dtype=torch.float32)
+        assert_close(dd, (d32o.double() * dloss).float(), atol=1e-10, name=f"dloss {dloss}")
+    loss3, _, none, _ = ops.fused_classifier(dev(x), dev(t), V, want_dlogits=False)
+    assert none is None and loss3.item() == loss.item()
+
+
+def test_cross_entropy_all_ignored_and_bad_targets(ops):
+    x = randn((6, 128), 115, dtype=torch.bfloat16)
+    t = torch.full((6,), -100, dtype=torch.int64)
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t), 100)
+    assert math.isnan(loss.item()) and tw.item() == 0 and (row == 0).all() and (d == 0).all()  # mean over nothing
+    t2 = torch.tensor([0, 99, 100, 5000, -7, 3], dtype=torch.int64)  # out-of-range targets count as ignored
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t2), 100)
+    assert tw.item() == 3 and (row[2:5] == 0).all() and (d[2:5] == 0).all() and math.isfinite(loss.item())
+
+
+def test_cross_entropy_config2_full_size(ops, co):
+    """Benchmark configuration 2: [8192, 50257] bf16, stride 50304, in place."""
+    N, V, stride = 8192, 50257, 50304
+    x = randn((N, stride), 1339, std=2.0, dtype=torch.bfloat16)
+    t = randint(0, V, (N,), 1340)
+    gx = dev(x)
+    loss, row, d, tw = ops.fused_classifier(gx, dev(t), V, inplace=True)
+    assert tw.item() == N
+    # size-independent properties
+    assert (gx[:, V:] == 0).all()
+    sums = gx[:, :V].float().sum(1)
+    assert sums.abs().max().item() < 2e-6  # (softmax - onehot)/N sums to 0 up to bf16 rounding of 50257 terms
+    assert abs(loss.item() - row.double().mean().item()) < 1e-5
+    assert (gx[torch.arange(N), dev(t)] < 0).all()  # p - 1 < 0 at the target
+    # the oracle on a sample of rows; dlogits of a row depends on the others only through 1/N
+    pick = torch.arange(0, N, 171)
+    _, row2, d2, _ = co.cross_entropy(x[pick], t[pick], V, reduction="sum", dloss=1.0 / N)
+    assert_close(row[pick], row2.float(), atol=1e-5, name="row loss sample")
+    assert_close(gx[pick], d2, atol=1e-10, name="dlogits sample")
