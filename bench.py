@@ -1,0 +1,378 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPT-2 training kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one fused-classifier call (row softmax + cross-entropy + in-place
+dlogits) on logits [8192, 50257] bf16 with row stride 50304 - the
+configuration the headline metric is quoted on.  W untimed steps, then exactly
+K timed steps between device synchronisations; one JSON line on stdout.
+
+The same line carries
+  roofline      the dominant kernel (the row pass) against the 8 TB/s HBM peak,
+                its duration measured with HIP events inside the timed region
+  per_op        every op of the hot path at its benchmark configuration:
+                ms, GB/s of algorithmic bytes and fraction of the HBM peak,
+                warm (same buffers) and cold (buffers rotated over > 512 MB so
+                the 256 MB Infinity Cache cannot serve them)
+  cpu_baseline  the reference's own op sequence on the ATen CPU backend
+                (oracle/aten_port.py), timed here on this box's host cores
+
+Inputs are synthetic (seeded normal logits, uniform targets) and resident in
+HBM before the timed region starts.  This build is single-GPU: --gpus above 1
+is refused.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+# benchmark configuration 2
+CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
+# algorithmic bytes per fused-classifier call: read the class columns of the logits once and
+# write them once (bf16), read the int64 targets, write fp32 row losses and the mean
+CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gpt2_param_sizes(n_layer, C, V=50257, T=1024):
+    sizes = [V * C, T * C]
+    for _ in range(n_layer):
+        sizes += [C, C, C * 3 * C, 3 * C, C * C, C, C, C, C * 4 * C, 4 * C, 4 * C * C, C]
+    return sizes + [C, C]
+
+
+def event_ms(fn, reps, torch):
+    """Median / mean duration of one call, each bracketed by its own pair of events."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    torch.cuda.synchronize()
+    for i in range(reps):
+        starts[i].record()
+        fn(i)
+        ends[i].record()
+    torch.cuda.synchronize()
+    ts = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    return statistics.median(ts), sum(ts) / len(ts)
+
+
+def run_headline(args, torch, ops, capi):
+    dev = torch.device("cuda:0")
+    lib = capi.load()
+    K, W = args.steps, args.warmup
+    n_buf = min(K + W, args.max_buffers)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1337 + 2)
+    master = (torch.randn((CE_N, CE_STRIDE), generator=g, device=dev, dtype=torch.float32) * 2.0).to(torch.bfloat16)
+    targets = torch.randint(0, CE_V, (CE_N,), generator=g, device=dev, dtype=torch.int64)
+    bufs = [master.clone() for _ in range(n_buf)]
+    row_loss = torch.empty(CE_N, dtype=torch.float32, device=dev)
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    tw = torch.empty((), dtype=torch.float32, device=dev)
+    ws_bytes = lib.cs_fused_classifier_workspace_bytes(CE_N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    P = ctypes.c_void_p
+
+    def phase(buf, which):
+        code = lib.cs_fused_classifier_phases(P(buf.data_ptr()), P(buf.data_ptr()), P(targets.data_ptr()),
+                                              P(row_loss.data_ptr()), P(loss.data_ptr()), P(tw.data_ptr()),
+                                              P(ws.data_ptr()), ws_bytes, CE_N, CE_V, CE_STRIDE, -100, capi.REDUCTION_MEAN,
+                                              1.0, capi.BF16, capi.BF16, which, stream)
+        capi.check("cs_fused_classifier_phases", code)
+
+    def step(i, ev=None):
+        buf = bufs[i % n_buf]
+        phase(buf, 1)
+        if ev:
+            ev[0].record()
+        phase(buf, 2)
+        if ev:
+            ev[1].record()
+        phase(buf, 4)
+
+    for i in range(W):
+        step(i)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(W + i, evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kernel_ms = [a.elapsed_time(b) for a, b in evs]
+    first_loss = loss.item()
+    reused = K + W > n_buf
+    return {
+        "seconds": t1 - t0,
+        "ms_per_step": (t1 - t0) / K * 1e3,
+        "rows_kernel_ms_avg": sum(kernel_ms) / K,
+        "rows_kernel_ms_median": statistics.median(kernel_ms),
+        "loss": first_loss,
+        "buffers": n_buf,
+        "buffers_reused": reused,
+    }
+
+
+def per_op_table(args, torch, ops):
+    """Every op at its benchmark configuration; returns a list of dicts."""
+    dev = torch.device("cuda:0")
+    reps = args.op_reps
+    g = torch.Generator(device=dev)
+    g.manual_seed(1337)
+    out = []
+
+    def randn(shape, std=1.0, mean=0.0, dtype=torch.bfloat16):
+        return (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean).to(dtype)
+
+    def add(name, config, nbytes, make_set, call):
+        """make_set() builds one set of buffers; call(set) issues the op once."""
+        n_cold = max(2, math.ceil(600e6 / nbytes) + 1)
+        n_cold = min(n_cold, 64)
+        sets = [make_set() for _ in range(n_cold)]
+        for s in sets[:2]:
+            call(s)
+        warm_med, warm_avg = event_ms(lambda i: call(sets[0]), reps, torch)
+        cold_med, cold_avg = event_ms(lambda i: call(sets[i % n_cold]), reps, torch)
+        rec = {
+            "op": name, "config": config, "algorithmic_bytes": nbytes,
+            "ms_warm": round(warm_med, 5), "ms_cold": round(cold_med, 5),
+            "gbps_warm": round(nbytes / warm_med / 1e6, 1), "gbps_cold": round(nbytes / cold_med / 1e6, 1),
+            "frac_cold": round(nbytes / cold_med / 1e6 / HBM_PEAK_GBPS, 4),
+            "buffer_sets": n_cold,
+        }
+        out.append(rec)
+        log(f"[per-op] {name:28s} {config:34s} warm {warm_med*1e3:9.1f} us  cold {cold_med*1e3:9.1f} us  "
+            f"{rec['gbps_cold']:8.1f} GB/s  {rec['frac_cold']*100:5.1f}% of HBM peak")
+        del sets
+        torch.cuda.empty_cache()
+
+    # ---- configuration 3: LayerNorm [8192,768] bf16, fp32 parameters
+    for tag, rows, C in (("small", 8192, 768), ("xl", 16384, 1600)):
+        gamma, beta = randn(C, 0.02, 1.0, torch.float32), randn(C, 0.02, 0.0, torch.float32)
+        fwd_bytes = 2 * rows * C * 2 + 2 * C * 4 + 2 * rows * 4
+        bwd_bytes = 3 * rows * C * 2 + 2 * rows * 4 + C * 4 + 2 * C * 4
+
+        def mk():
+            x = randn((rows, C))
+            y, mean, rstd = ops.layernorm_forward(x, gamma, beta, 1e-5)
+            return {"x": x, "dy": randn((rows, C)), "mean": mean, "rstd": rstd}
+
+        add("layernorm_fwd", f"{tag} [{rows},{C}] bf16", fwd_bytes, mk,
+            lambda s: ops.layernorm_forward(s["x"], gamma, beta, 1e-5))
+        add("layernorm_bwd", f"{tag} [{rows},{C}] bf16", bwd_bytes, mk,
+            lambda s: ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma))
+
+    # ---- configuration 3: GeLU [8192,3072] bf16, tanh (benchmark) and erf (the reference's form)
+    n = 8192 * 3072
+    for mode in ("tanh", "none"):
+        def mk():
+            return {"x": randn(n, 1.5), "dy": randn(n)}
+
+        label = "tanh" if mode == "tanh" else "erf"
+        add(f"gelu_fwd_{label}", "[8192,3072] bf16", 2 * n * 2, mk, lambda s: ops.gelu_forward(s["x"], mode))
+        add(f"gelu_bwd_{label}", "[8192,3072] bf16", 3 * n * 2, mk, lambda s: ops.gelu_backward(s["dy"], s["x"], mode))
+
+    # ---- configuration 1: token + position embedding
+    V, T = 50257, 1024
+    for tag, B, C in (("small", 8, 768), ("xl", 16, 1600)):
+        wte, wpe = randn((V, C), 0.02), randn((T, C), 0.02)
+        ranks = torch.arange(1, V + 1, dtype=torch.float64, device=dev).pow(-1.1)
+        for kind in ("uniform", "zipf"):
+            if tag == "xl" and kind == "uniform":
+                continue
+            if kind == "uniform":
+                ids = torch.randint(0, V, (B, T), generator=g, device=dev, dtype=torch.int64)
+            else:
+                ids = torch.multinomial(ranks / ranks.sum(), B * T, replacement=True, generator=g).reshape(B, T)
+            fwd_bytes = B * T * 8 + B * T * C * 2 + T * C * 2 + B * T * C * 2
+            bwd_bytes = B * T * 8 + B * T * C * 2 + V * C * 2 + T * C * 2
+
+            def mk():
+                return {"dout": randn((B, T, C))}
+
+            add("embedding_fwd", f"{tag} {kind} B{B} T{T} C{C}", fwd_bytes, mk,
+                lambda s: ops.embedding_forward_add(wte, wpe, ids))
+            add("embedding_bwd", f"{tag} {kind} B{B} T{T} C{C}", bwd_bytes, mk,
+                lambda s: ops.embedding_backward_fused(s["dout"], ids, V))
+        del wte, wpe
+
+    # ---- configuration 0 / 4: AdamW over the GPT-2-small / XL parameter sets, one launch
+    for tag, n_layer, C in (("small", 12, 768), ("xl", 48, 1600)):
+        sizes = gpt2_param_sizes(n_layer, C)
+        total = sum(sizes)
+        if tag == "xl" and not args.xl_adamw:
+            continue
+        w = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 0.02, generator=g)
+        grad = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 1e-3, generator=g)
+        offs = [0]
+        for s in sizes:
+            offs.append(offs[-1] + s)
+        ws_ = [w[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+        gs_ = [grad[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+        opt = ops.MultiTensorAdamW(ws_, gs_, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+        opt.step()
+        med, avg = event_ms(lambda i: opt.step(), reps, torch)
+        nbytes = 28 * total
+        rec = {"op": "adamw_multi_tensor", "config": f"{tag} {len(sizes)} tensors {total} fp32 params",
+               "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
+               "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
+               "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1}
+        out.append(rec)
+        log(f"[per-op] adamw_multi_tensor           {tag:34s} {med*1e3:9.1f} us  {rec['gbps_cold']:8.1f} GB/s  "
+            f"{rec['frac_cold']*100:5.1f}% of HBM peak")
+        if tag == "small":
+            # the reference's launch shape: one launch per tensor (src/module/adamw.cpp:32-38)
+            ms_, vs_ = [torch.zeros_like(x) for x in ws_], [torch.zeros_like(x) for x in ws_]
+
+            def per_tensor(i):
+                for a, b, c, d in zip(ws_, gs_, ms_, vs_):
+                    ops.adamw_step(a, b, c, d, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, t=1)
+
+            per_tensor(0)
+            med2, _ = event_ms(per_tensor, max(3, reps // 4), torch)
+            out.append({"op": "adamw_per_tensor_launches", "config": f"{tag} {len(sizes)} launches",
+                        "algorithmic_bytes": nbytes, "ms_warm": round(med2, 5), "ms_cold": round(med2, 5),
+                        "gbps_warm": round(nbytes / med2 / 1e6, 1), "gbps_cold": round(nbytes / med2 / 1e6, 1),
+                        "frac_cold": round(nbytes / med2 / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1})
+            log(f"[per-op] adamw, {len(sizes)} launches      {tag:34s} {med2*1e3:9.1f} us")
+            del ms_, vs_
+        del opt, w, grad, ws_, gs_
+        torch.cuda.empty_cache()
+
+    # ---- configuration 4: XL fused classifier [16384, 50257]
+    if args.xl_ce:
+        N = 16384
+        x = randn((N, CE_STRIDE), 2.0)
+        t = torch.randint(0, CE_V, (N,), generator=g, device=dev, dtype=torch.int64)
+        nbytes = 2 * N * CE_V * 2 + N * 12 + 4
+        bufs = [x.clone() for _ in range(3)]
+        ops.fused_classifier(bufs[0], t, CE_V, inplace=True)
+        med, avg = event_ms(lambda i: ops.fused_classifier(bufs[i % 3], t, CE_V, inplace=True), max(5, reps // 4), torch)
+        out.append({"op": "fused_classifier", "config": f"xl [{N},{CE_V}] bf16 stride {CE_STRIDE}",
+                    "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
+                    "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
+                    "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 3})
+        log(f"[per-op] fused_classifier xl          {med*1e3:9.1f} us  {nbytes/med/1e6:8.1f} GB/s")
+    return out
+
+
+def cpu_baseline(args, torch):
+    """The reference's cross-entropy op sequence on the ATen CPU backend, full configuration-2 size."""
+    from oracle import aten_port as ap
+
+    rows = args.cpu_rows
+    g = torch.Generator().manual_seed(1337 + 2)
+    # the values the GPU sees: bf16 logits, widened to fp32 as the reference's AMP path does
+    x = (torch.randn((rows, CE_V), generator=g) * 2.0).to(torch.bfloat16).float()
+    t = torch.randint(0, CE_V, (rows,), generator=g)
+    times = []
+    for i in range(1 + args.cpu_reps):
+        t0 = time.perf_counter()
+        loss, grad, _ = ap.cross_entropy(x, t)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times[1:])
+    nbytes = CE_BYTES * rows / CE_N
+    return {
+        "value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{rows} of {CE_N} rows x {CE_V} classes, fp32-widened bf16 logits; at::log_softmax + nll_loss_forward + "
+                  f"nll_loss_backward + _log_softmax_backward_data on the ATen CPU backend; median of {args.cpu_reps} "
+                  f"after 1 warm-up; {med*1e3:.1f} ms per call; same algorithmic bytes per row as the GPU figure",
+        "ms": round(med * 1e3, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--op-reps", type=int, default=40, help="timed calls per op in the per-op table")
+    ap.add_argument("--max-buffers", type=int, default=32, help="distinct logits buffers rotated by the headline loop")
+    ap.add_argument("--no-per-op", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-xl-adamw", dest="xl_adamw", action="store_false", help="skip the 25 GB XL AdamW line")
+    ap.add_argument("--no-xl-ce", dest="xl_ce", action="store_false")
+    ap.add_argument("--cpu-rows", type=int, default=CE_N)
+    ap.add_argument("--cpu-reps", type=int, default=5)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (no collectives are part of it); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device visible; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    from core_scheduler_amd import _capi as capi
+    from core_scheduler_amd import ops
+
+    capi.load()  # raises if the kernel library is not built
+    log(f"[bench] device: {torch.cuda.get_device_name(0)}; torch {torch.__version__}")
+
+    head = run_headline(args, torch, ops, capi)
+    achieved = CE_BYTES / (head["rows_kernel_ms_avg"] * 1e-3) / 1e9
+    value = CE_BYTES * args.steps / head["seconds"] / 1e9
+    log(f"[bench] fused classifier: {head['ms_per_step']:.4f} ms/step wall, row kernel {head['rows_kernel_ms_avg']:.4f} ms "
+        f"(events), {achieved:.0f} GB/s = {achieved / HBM_PEAK_GBPS * 100:.1f}% of HBM peak, loss {head['loss']:.4f}")
+
+    table = [] if args.no_per_op else per_op_table(args, torch, ops)
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(args, torch)
+        log(f"[bench] CPU baseline (ATen CPU, {cpu['cores']} threads): {cpu['ms']:.1f} ms, {cpu['value']} GB/s")
+
+    line = {
+        "metric": "fused CE HBM GB/s at 8192x50257 bf16 (ms in ms_per_step; every op in per_op)",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "fused classifier (softmax + cross-entropy + in-place dlogits), logits [8192, 50257] bf16, "
+                        "row stride 50304, int64 targets, mean reduction (BASELINE configs[2])",
+            "algorithmic_bytes_per_step": CE_BYTES,
+            "logits_buffers_rotated": head["buffers"],
+            "loss": round(head["loss"], 5),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "ce_rows_kernel<bf16, bf16, 1024, 7>",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "kernel_ms_avg": round(head["rows_kernel_ms_avg"], 5),
+            "kernel_ms_median": round(head["rows_kernel_ms_median"], 5),
+            "traffic": None,
+        },
+        "cpu_baseline": cpu,
+        "per_op": table,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -86,6 +86,10 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 7 + [c_size_t] + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_void_p],
     ),
+    "cs_fused_classifier_phases": (
+        c_int,
+        [c_void_p] * 7 + [c_size_t] + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_int, c_void_p],
+    ),
 }
 
 _lib = None

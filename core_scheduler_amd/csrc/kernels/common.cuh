@@ -114,15 +114,61 @@ struct MaxOp {
   }
 };
 
-// Butterfly over the 64 lanes of a wavefront; every lane ends with the full
-// result and the combination order is fixed, so results are reproducible.
+// Butterfly over the 64 lanes of a wavefront through the LDS crossbar
+// (ds_bpermute); every lane ends with the full result and the combination
+// order is fixed, so results are reproducible.  Works for any 4/8-byte type.
 template <typename A, typename Op>
-__device__ __forceinline__ A wave_reduce(A v, Op op) {
+__device__ __forceinline__ A wave_reduce_generic(A v, Op op) {
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) {
     v = op(v, __shfl_xor(v, off, kWave));
   }
   return v;
+}
+
+// DPP lane exchanges inside a row of 16 lanes: no LDS traffic, a few cycles.
+// All 64 lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+  return __builtin_bit_cast(float, r);
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7-i inside each 8
+constexpr int kDppRowMirror = 0x140;   // lane i <-> 15-i inside each 16
+
+// fp32 wavefront all-reduce: four DPP steps give every lane its row's
+// result, four v_readlane + three ops fold the four rows.  Fixed order.
+template <typename Op>
+__device__ __forceinline__ float wave_reduce(float v, Op op) {
+  v = op(v, dpp_f32<kDppQuadXor1>(v));
+  v = op(v, dpp_f32<kDppQuadXor2>(v));
+  v = op(v, dpp_f32<kDppHalfMirror>(v));
+  v = op(v, dpp_f32<kDppRowMirror>(v));
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return op(op(r0, r1), op(r2, r3));
+}
+template <typename Op>
+__device__ __forceinline__ int wave_reduce(int v, Op op) {
+  v = op(v, dpp_i32<kDppQuadXor1>(v));
+  v = op(v, dpp_i32<kDppQuadXor2>(v));
+  v = op(v, dpp_i32<kDppHalfMirror>(v));
+  v = op(v, dpp_i32<kDppRowMirror>(v));
+  const int r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+  const int r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+  return op(op(r0, r1), op(r2, r3));
+}
+template <typename Op>
+__device__ __forceinline__ double wave_reduce(double v, Op op) {
+  return wave_reduce_generic(v, op);
 }
 
 // Workgroup reduction through LDS.  `scratch` holds one A per wavefront.

@@ -198,6 +198,167 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
   }
 }
 
+// Streaming variant for wide rows (the GPT-2 vocabulary): one 1024-lane
+// workgroup per CU walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and
+// loads the next row into a second register set before it starts on the
+// current one, so the CU's memory pipe stays busy while its VALUs work; the
+// stores of a finished row drain under the next row's arithmetic.  Without
+// this, all workgroups load, compute and store in lockstep and HBM idles for
+// the whole compute phase.
+//
+// Each element costs one hardware exp2: lane-local max first, then
+// e = 2^((x - m_lane) log2e) is kept in registers, one exchange of (max, sum)
+// pairs across the 16 waves gives the row's max and sum, and the output is
+// e * f with one per-lane factor f = 2^(m_lane*log2e - log2(sum) - max*log2e) * s.
+template <typename T, typename TD, int VPT>
+__global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
+    const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
+    const int *__restrict__ ws_count, int64_t N, int64_t V, int64_t row_stride,
+    int64_t ignore_index, int reduction, float dloss) {
+  constexpr int BLOCK = 1024;
+  constexpr int VN = Vec16<T>::n;
+  constexpr int kWaves = BLOCK / kWave;
+  __shared__ float red_m[2][kWaves], red_s[2][kWaves];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int nvec = (int)(row_stride / VN);
+  const int iV = (int)V;
+
+  float scale = dloss;
+  if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
+  const float log2_scale = __builtin_amdgcn_logf(fabsf(scale));  // -inf for 0: every output 0
+  const bool negate = scale < 0.f;
+
+  int64_t row = blockIdx.x;
+  Vec16<T> cur[VPT];
+  int64_t tgt = 0;
+  bool live = false;
+  float x_t = 0.f;
+  if (row < N) {
+    tgt = targets[row];
+    live = target_counts(tgt, V, ignore_index);
+    if (live) {
+      const T *x = logits + row * row_stride;
+#pragma unroll
+      for (int j = 0; j < VPT; ++j) {
+        const int idx = tid + BLOCK * j;
+        if (idx < nvec) cur[j] = load16_stream(x + (int64_t)idx * VN);
+      }
+      if (tid == 0) x_t = to_acc(x[tgt]);
+    }
+  }
+  int parity = 0;
+  while (row < N) {
+    // ---- issue the next row's loads
+    const int64_t nrow = row + gridDim.x;
+    Vec16<T> nxt[VPT];
+    int64_t ntgt = 0;
+    bool nlive = false;
+    float nx_t = 0.f;
+    if (nrow < N) {
+      ntgt = targets[nrow];
+      nlive = target_counts(ntgt, V, ignore_index);
+      if (nlive) {
+        const T *x = logits + nrow * row_stride;
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+          const int idx = tid + BLOCK * j;
+          if (idx < nvec) nxt[j] = load16_stream(x + (int64_t)idx * VN);
+        }
+        if (tid == 0) nx_t = to_acc(x[ntgt]);
+      }
+    }
+
+    if (!live) {
+      if (tid == 0 && row_loss) row_loss[row] = 0.f;
+      if (dlogits) {
+        float z[VN];
+#pragma unroll
+        for (int k = 0; k < VN; ++k) z[k] = 0.f;
+        for (int idx = tid; idx < nvec; idx += BLOCK)
+          store_out<T, TD, VN>(dlogits + row * row_stride + (int64_t)idx * VN, z);
+      }
+    } else {
+      // ---- widen, mask what is not a class column to -inf, lane-local max
+      float e[VPT][VN];
+      float m = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < VPT; ++j) {
+        const int c0 = (tid + BLOCK * j) * VN;
+        if (c0 + VN <= iV) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k) {
+            e[j][k] = to_acc(cur[j].e[k]);
+            m = fmaxf(m, e[j][k]);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < VN; ++k) {
+            e[j][k] = c0 + k < iV ? to_acc(cur[j].e[k]) : -INFINITY;
+            m = fmaxf(m, e[j][k]);
+          }
+        }
+      }
+      // a lane without any class column: any finite stand-in keeps 2^(-inf - m) = 0
+      const float ml2 = (m == -INFINITY ? 0.f : m) * kLog2e;
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          e[j][k] = __builtin_amdgcn_exp2f(e[j][k] * kLog2e - ml2);
+          s += e[j][k];
+        }
+      // ---- (max, sum) across the wave, then across the 16 waves
+      const float mw2 = wave_reduce(ml2, MaxOp{});
+      const float sw = wave_reduce(s * __builtin_amdgcn_exp2f(ml2 - mw2), SumOp{});
+      if (lane == 0) {
+        red_m[parity][wave] = mw2;
+        red_s[parity][wave] = sw;
+      }
+      __syncthreads();
+      const float pm = lane < kWaves ? red_m[parity][lane] : -INFINITY;
+      const float ps = lane < kWaves ? red_s[parity][lane] : 0.f;
+      const float M2 = wave_reduce(pm, MaxOp{});
+      const float S = wave_reduce(ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
+      parity ^= 1;  // the other pair of arrays next time: one barrier per row is enough
+      const float log2_S = __builtin_amdgcn_logf(S);
+      if (tid == 0 && row_loss) row_loss[row] = (M2 + log2_S) * kLn2 - x_t;
+
+      if (dlogits) {
+        // a lane that holds no class column has e = 0 everywhere; give it f = 0 so that
+        // 0 * f cannot meet an overflowed factor
+        float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml2 - M2 - log2_S + log2_scale);
+        f = negate ? -f : f;
+        const int t_vec = (int)(tgt / VN), t_sub = (int)(tgt % VN);
+        TD *d = dlogits + row * row_stride;
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+          const int idx = tid + BLOCK * j;
+          if (idx < nvec) {
+            float o[VN];
+#pragma unroll
+            for (int k = 0; k < VN; ++k) o[k] = e[j][k] * f;
+            if (idx == t_vec) {
+#pragma unroll
+              for (int k = 0; k < VN; ++k)
+                if (k == t_sub) o[k] -= scale;
+            }
+            store_out<T, TD, VN>(d + (int64_t)idx * VN, o);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) cur[j] = nxt[j];
+    live = nlive;
+    tgt = ntgt;
+    x_t = nx_t;
+    row = nrow;
+  }
+}
+
 // Any V, stride and alignment; fp64 too.  Three sweeps over the row, the
 // later ones served by the cache.
 template <typename T, typename TD>
@@ -243,6 +404,20 @@ __global__ __launch_bounds__(256) void ce_rows_general_kernel(
   }
 }
 
+// CUs of the current device, asked once per device.
+int64_t compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 template <typename T, typename TD>
 int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
                 const int *ws_count, int64_t N, int64_t V, int64_t row_stride,
@@ -262,10 +437,19 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         CS_CE(64, 8);
       } else if (nvec <= 256 * 8) {
         CS_CE(256, 8);
-      } else if (nvec <= 1024 * 7) {
-        CS_CE(1024, 7);
       } else if (nvec <= 1024 * 8) {
-        CS_CE(1024, 8);
+        // one persistent workgroup per CU
+        const int64_t cus = compute_units();
+        const dim3 pgrid((unsigned)(N < cus ? N : cus));
+        if (nvec <= 1024 * 7) {
+          ce_rows_stream_kernel<T, TD, 7><<<pgrid, dim3(1024), 0, s>>>(
+              (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,
+              ignore_index, reduction, dloss);
+        } else {
+          ce_rows_stream_kernel<T, TD, 8><<<pgrid, dim3(1024), 0, s>>>(
+              (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,
+              ignore_index, reduction, dloss);
+        }
       } else {
         CS_CE(1024, 16);
       }
@@ -290,46 +474,70 @@ extern "C" size_t cs_fused_classifier_workspace_bytes(int64_t N) {
   return kWsHeader + ((size_t)N * sizeof(float) + 255) / 256 * 256;
 }
 
-extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int64_t *targets,
-                                   float *row_loss, float *loss, float *total_weight,
-                                   void *workspace, size_t workspace_bytes, int64_t N, int64_t V,
-                                   int64_t row_stride, int64_t ignore_index, int reduction,
-                                   float dloss, int dtype, int dlogits_dtype, void *stream) {
-  if (N < 0 || V <= 0 || row_stride < V) return CS_ERR_INVALID_ARGUMENT;
-  if (reduction != CS_REDUCTION_NONE && reduction != CS_REDUCTION_MEAN &&
-      reduction != CS_REDUCTION_SUM)
-    return CS_ERR_INVALID_ARGUMENT;
-  const size_t es = dtype_size(dtype), ds = dtype_size(dlogits_dtype);
-  if (es == 0 || ds == 0) return CS_ERR_UNSUPPORTED;
-  if (dlogits_dtype != dtype && !(dlogits_dtype == CS_F32 && es == 2)) return CS_ERR_UNSUPPORTED;
-  if (N > 0x7fffffffLL || V > 0x7fffffffLL || row_stride > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
-  if (!workspace || workspace_bytes < cs_fused_classifier_workspace_bytes(N) ||
-      !aligned_to(workspace, 256))
-    return CS_ERR_WORKSPACE;
-  if (reduction == CS_REDUCTION_NONE && !row_loss) return CS_ERR_INVALID_ARGUMENT;
-  if (reduction != CS_REDUCTION_NONE && !loss) return CS_ERR_INVALID_ARGUMENT;
-  if (N > 0 && (!logits || !targets)) return CS_ERR_INVALID_ARGUMENT;
-  if ((logits && !aligned_to(logits, es)) || (dlogits && !aligned_to(dlogits, ds)) ||
-      (targets && !aligned_to(targets, 8)) || (row_loss && !aligned_to(row_loss, 4)) ||
-      (loss && !aligned_to(loss, 4)) || (total_weight && !aligned_to(total_weight, 4)))
-    return CS_ERR_MISALIGNED;
-  if (dlogits == logits && dlogits_dtype != dtype) return CS_ERR_INVALID_ARGUMENT;
+namespace {
 
+struct CeArgs {
+  const void *logits;
+  void *dlogits;
+  const int64_t *targets;
+  float *row_loss;
+  float *loss;
+  float *total_weight;
+  void *workspace;
+  size_t workspace_bytes;
+  int64_t N, V, row_stride, ignore_index;
+  int reduction;
+  float dloss;
+  int dtype, dlogits_dtype;
+};
+
+int ce_validate(const CeArgs &a) {
+  if (a.N < 0 || a.V <= 0 || a.row_stride < a.V) return CS_ERR_INVALID_ARGUMENT;
+  if (a.reduction != CS_REDUCTION_NONE && a.reduction != CS_REDUCTION_MEAN &&
+      a.reduction != CS_REDUCTION_SUM)
+    return CS_ERR_INVALID_ARGUMENT;
+  const size_t es = dtype_size(a.dtype), ds = dtype_size(a.dlogits_dtype);
+  if (es == 0 || ds == 0) return CS_ERR_UNSUPPORTED;
+  if (a.dlogits_dtype != a.dtype && !(a.dlogits_dtype == CS_F32 && es == 2))
+    return CS_ERR_UNSUPPORTED;
+  if (a.N > 0x7fffffffLL || a.V > 0x7fffffffLL || a.row_stride > 0x7fffffffLL)
+    return CS_ERR_TOO_LARGE;
+  if (!a.workspace || a.workspace_bytes < cs_fused_classifier_workspace_bytes(a.N) ||
+      !aligned_to(a.workspace, 256))
+    return CS_ERR_WORKSPACE;
+  if (a.reduction == CS_REDUCTION_NONE && !a.row_loss) return CS_ERR_INVALID_ARGUMENT;
+  if (a.reduction != CS_REDUCTION_NONE && !a.loss) return CS_ERR_INVALID_ARGUMENT;
+  if (a.N > 0 && (!a.logits || !a.targets)) return CS_ERR_INVALID_ARGUMENT;
+  if ((a.logits && !aligned_to(a.logits, es)) || (a.dlogits && !aligned_to(a.dlogits, ds)) ||
+      (a.targets && !aligned_to(a.targets, 8)) || (a.row_loss && !aligned_to(a.row_loss, 4)) ||
+      (a.loss && !aligned_to(a.loss, 4)) || (a.total_weight && !aligned_to(a.total_weight, 4)))
+    return CS_ERR_MISALIGNED;
+  if (a.dlogits == a.logits && a.dlogits_dtype != a.dtype) return CS_ERR_INVALID_ARGUMENT;
+  return CS_OK;
+}
+
+// phases: 1 = count the rows that are not ignored, 2 = the row pass,
+// 4 = reduce the row losses
+int ce_run(const CeArgs &a, int phases, void *stream) {
+  int st = ce_validate(a);
+  if (st != CS_OK) return st;
   hipStream_t s = as_stream(stream);
-  char *ws = static_cast<char *>(workspace);
+  char *ws = static_cast<char *>(a.workspace);
   int *ws_count = reinterpret_cast<int *>(ws);
   float *ws_weight = reinterpret_cast<float *>(ws) + 1;
-  float *rows = row_loss ? row_loss : reinterpret_cast<float *>(ws + kWsHeader);
-
-  ce_count_kernel<<<dim3(1), dim3(1024), 0, s>>>(targets, N, V, ignore_index, ws_count, ws_weight);
-  int st = launch_status();
-  if (st != CS_OK) return st;
-  if (N > 0) {
-#define CS_CALL(T, TD)                                                                     \
-  st = launch_rows<T, TD>(logits, dlogits, targets, rows, ws_count, N, V, row_stride,      \
-                          ignore_index, reduction, dloss, s)
-    const bool wide = dlogits_dtype != dtype;
-    switch (dtype) {
+  float *rows = a.row_loss ? a.row_loss : reinterpret_cast<float *>(ws + kWsHeader);
+  if (phases & 1) {
+    ce_count_kernel<<<dim3(1), dim3(1024), 0, s>>>(a.targets, a.N, a.V, a.ignore_index, ws_count,
+                                                   ws_weight);
+    st = launch_status();
+    if (st != CS_OK) return st;
+  }
+  if ((phases & 2) && a.N > 0) {
+#define CS_CALL(T, TD)                                                                      \
+  st = launch_rows<T, TD>(a.logits, a.dlogits, a.targets, rows, ws_count, a.N, a.V,         \
+                          a.row_stride, a.ignore_index, a.reduction, a.dloss, s)
+    const bool wide = a.dlogits_dtype != a.dtype;
+    switch (a.dtype) {
       case CS_F32: CS_CALL(float, float); break;
       case CS_F64: CS_CALL(double, double); break;
       case CS_F16:
@@ -350,8 +558,38 @@ extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int6
 #undef CS_CALL
     if (st != CS_OK) return st;
   }
-  ce_reduce_kernel<<<dim3(1), dim3(1024), 0, s>>>(rows, N, ws_count, reduction,
-                                                  reduction == CS_REDUCTION_NONE ? nullptr : loss,
-                                                  total_weight);
-  return launch_status();
+  if (phases & 4) {
+    ce_reduce_kernel<<<dim3(1), dim3(1024), 0, s>>>(
+        rows, a.N, ws_count, a.reduction, a.reduction == CS_REDUCTION_NONE ? nullptr : a.loss,
+        a.total_weight);
+    st = launch_status();
+  }
+  return st;
+}
+
+}  // namespace
+
+extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int64_t *targets,
+                                   float *row_loss, float *loss, float *total_weight,
+                                   void *workspace, size_t workspace_bytes, int64_t N, int64_t V,
+                                   int64_t row_stride, int64_t ignore_index, int reduction,
+                                   float dloss, int dtype, int dlogits_dtype, void *stream) {
+  const CeArgs a{logits, dlogits, targets,      row_loss,  loss,  total_weight, workspace,
+                 workspace_bytes, N, V, row_stride, ignore_index, reduction, dloss, dtype,
+                 dlogits_dtype};
+  return ce_run(a, 1 | 2 | 4, stream);
+}
+
+extern "C" int cs_fused_classifier_phases(const void *logits, void *dlogits,
+                                          const int64_t *targets, float *row_loss, float *loss,
+                                          float *total_weight, void *workspace,
+                                          size_t workspace_bytes, int64_t N, int64_t V,
+                                          int64_t row_stride, int64_t ignore_index, int reduction,
+                                          float dloss, int dtype, int dlogits_dtype, int phases,
+                                          void *stream) {
+  if (phases <= 0 || phases > 7) return CS_ERR_INVALID_ARGUMENT;
+  const CeArgs a{logits, dlogits, targets,      row_loss,  loss,  total_weight, workspace,
+                 workspace_bytes, N, V, row_stride, ignore_index, reduction, dloss, dtype,
+                 dlogits_dtype};
+  return ce_run(a, phases, stream);
 }

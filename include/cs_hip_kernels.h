@@ -244,6 +244,26 @@ int cs_fused_classifier(const void *logits, void *dlogits,
                         int reduction, float dloss, int dtype,
                         int dlogits_dtype, void *stream);
 
+/* The same call split into its three launches, for callers that want to
+ * time or capture them apart, or that already know the row count:
+ * phases is a bit set of CS_CE_PHASE_COUNT (write the number of rows that are
+ * not ignored into the workspace), CS_CE_PHASE_ROWS (the pass over the logits;
+ * needs the count in the workspace) and CS_CE_PHASE_REDUCE (row losses ->
+ * loss, total_weight).  All three in one call is cs_fused_classifier. */
+enum cs_ce_phase {
+  CS_CE_PHASE_COUNT = 1,
+  CS_CE_PHASE_ROWS = 2,
+  CS_CE_PHASE_REDUCE = 4,
+};
+int cs_fused_classifier_phases(const void *logits, void *dlogits,
+                               const int64_t *targets, float *row_loss,
+                               float *loss, float *total_weight,
+                               void *workspace, size_t workspace_bytes,
+                               int64_t N, int64_t V, int64_t row_stride,
+                               int64_t ignore_index, int reduction,
+                               float dloss, int dtype, int dlogits_dtype,
+                               int phases, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
