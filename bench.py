@@ -55,11 +55,30 @@ def gpt2_param_sizes(n_layer, C, V=50257, T=1024):
     return sizes + [C, C]
 
 
+_BLOCKER = {}
+
+
+def hold_gpu(torch, ms=3.0):
+    """Queues ~`ms` of plain copies so that the launches that follow are all enqueued while the
+    GPU is still busy: the timed calls then run back to back, as they do inside a training step,
+    instead of each waiting for the host to issue it."""
+    from core_scheduler_amd import _capi
+
+    if "buf" not in _BLOCKER:
+        _BLOCKER["buf"] = (torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0"),
+                           torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0"))
+    a, b = _BLOCKER["buf"]
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(max(1, int(ms / 0.35))):  # 1 GiB each way takes ~0.35 ms
+        _capi.load().cs_stream_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), 1 << 30, st)
+
+
 def event_ms(fn, reps, torch):
     """Median / mean duration of one call, each bracketed by its own pair of events."""
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
     torch.cuda.synchronize()
+    hold_gpu(torch)
     for i in range(reps):
         starts[i].record()
         fn(i)
@@ -138,8 +157,15 @@ def per_op_table(args, torch, ops):
     def randn(shape, std=1.0, mean=0.0, dtype=torch.bfloat16):
         return (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean).to(dtype)
 
+    only = [o for o in args.ops.split(",") if o]
+
+    def wanted(name):
+        return not only or any(name.startswith(o) for o in only)
+
     def add(name, config, nbytes, make_set, call):
         """make_set() builds one set of buffers; call(set) issues the op once."""
+        if not wanted(name):
+            return
         n_cold = max(2, math.ceil(600e6 / nbytes) + 1)
         n_cold = min(n_cold, 64)
         sets = [make_set() for _ in range(n_cold)]
@@ -214,7 +240,7 @@ def per_op_table(args, torch, ops):
     for tag, n_layer, C in (("small", 12, 768), ("xl", 48, 1600)):
         sizes = gpt2_param_sizes(n_layer, C)
         total = sum(sizes)
-        if tag == "xl" and not args.xl_adamw:
+        if (tag == "xl" and not args.xl_adamw) or not wanted("adamw"):
             continue
         w = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 0.02, generator=g)
         grad = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 1e-3, generator=g)
@@ -254,7 +280,7 @@ def per_op_table(args, torch, ops):
         torch.cuda.empty_cache()
 
     # ---- configuration 4: XL fused classifier [16384, 50257]
-    if args.xl_ce:
+    if args.xl_ce and wanted("fused_classifier"):
         N = 16384
         x = randn((N, CE_STRIDE), 2.0)
         t = torch.randint(0, CE_V, (N,), generator=g, device=dev, dtype=torch.int64)
@@ -304,6 +330,7 @@ def main():
     ap.add_argument("--op-reps", type=int, default=40, help="timed calls per op in the per-op table")
     ap.add_argument("--max-buffers", type=int, default=32, help="distinct logits buffers rotated by the headline loop")
     ap.add_argument("--no-per-op", action="store_true")
+    ap.add_argument("--ops", default="", help="comma list of op-name prefixes to keep in the per-op table")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-xl-adamw", dest="xl_adamw", action="store_false", help="skip the 25 GB XL AdamW line")
     ap.add_argument("--no-xl-ce", dest="xl_ce", action="store_false")

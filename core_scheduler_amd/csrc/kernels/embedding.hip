@@ -7,24 +7,31 @@
 //            were never indexed are zero            (src/compute/embedding.cpp:147-157)
 // positions: dwpe[t,:] (+)= sum_b dout[b,t,:]           (gpt2_single_device.cpp:565-566)
 //
-// The backward does not use floating point atomics.  It sorts (id, position)
-// keys, so equal ids become one contiguous segment in ascending position
-// order, and adds each segment's rows in that order in fp32, which makes the
-// result independent of scheduling:
-//   1. tile sort   - each workgroup bitonic-sorts a tile of keys in LDS
-//   2. merge rank  - every key finds its global rank by binary search in the
-//                    other tiles, is scattered to its place, and the first
-//                    key of every id marks its row in a bitmap
-//   3. window sums - one wavefront per 8 consecutive sorted entries adds the
-//                    runs of equal ids it sees; a run that is a whole segment
-//                    is written to its row, a run cut by the window edge is
-//                    left as an fp32 partial row
-//   4. finish      - segments longer than a window add their partial rows in
-//                    window order; in the same launch the rows whose bit is
-//                    clear are zero-filled and the position table gradient is
-//                    summed
-// The traffic that matters is step 4's dense write of dweight (V*C elements)
-// and one read of dout.
+// The backward uses no floating point atomics.  It sorts (id, position) keys,
+// so equal ids become one contiguous segment in ascending position order, and
+// adds each segment's rows in a fixed order in fp32, which makes the result
+// independent of scheduling.  Four launches:
+//   1. tile sort  - each workgroup bitonic-sorts 1024 keys, one per lane:
+//                   exchanges below 64 lanes are wave shuffles, the rest go
+//                   through LDS.  Spare workgroups of the same launch clear
+//                   the row bitmap and sum the position-table gradient, which
+//                   needs no order.
+//   2. merge rank - every key finds its global rank by binary search in the
+//                   other tiles (staged in LDS), is scattered to its place,
+//                   and the first key of every id marks its row in a bitmap.
+//   3. reduce     - a segmented sum.  A workgroup owns 64 consecutive sorted
+//                   entries, each of its 16 waves owns 4 of them and loads
+//                   their rows at once.  Runs of equal ids inside a wave are
+//                   added in registers; runs that cross waves are folded
+//                   through LDS in wave order; a segment that crosses
+//                   workgroups leaves one fp32 partial row per workgroup, so
+//                   a hot row is read by as many CUs as it has windows.
+//                   Further workgroups of the same launch zero the rows
+//                   whose bitmap bit is clear.
+//   4. finish     - the workgroup of a crossing segment's first window adds
+//                   that segment's partial rows in window order.
+// The traffic that matters is the dense write of dweight (V*C elements) and
+// one read of dout.
 #include "common.cuh"
 
 #include <type_traits>
@@ -33,11 +40,6 @@ namespace cs_hip {
 namespace {
 
 constexpr int kThreads = 256;
-
-template <typename IdxT>
-__device__ __forceinline__ int64_t load_index(const void *ids, int64_t i) {
-  return (int64_t) static_cast<const IdxT *>(ids)[i];
-}
 
 // ------------------------------------------------------------------ forward
 // One 16-byte vector per thread step; `nvec` vectors per row.
@@ -135,173 +137,266 @@ struct KeyCodec<uint64_t> {
   __device__ static uint32_t pos(uint64_t key, int) { return (uint32_t)key; }
 };
 
-constexpr int kTile = 2048;         // keys per sorted tile
-constexpr int kSortThreads = 1024;  // one compare-exchange pair per thread
+constexpr int kTile = 1024;  // keys per sorted tile = lanes of the sorting workgroup
 constexpr uint32_t kNoId = 0xFFFFFFFFu;
+constexpr int kWindow = 64;  // sorted entries per reducing workgroup
 
-// Blocks [0, n_tiles): sort one tile.  Blocks beyond: clear the row bitmap and
-// preset sorted_id to "no id" so unused tail slots are recognisable.
-template <typename KeyT, typename IdxT>
-__global__ __launch_bounds__(kSortThreads) void emb_bwd_tile_sort_kernel(
+// Position-table gradient for one 16-byte vector: dwpe[t, :] (+)= sum_b dout[b, t, :].
+template <typename T>
+__device__ __forceinline__ void positions_vector(const T *__restrict__ dout, T *__restrict__ dwpe,
+                                                 int64_t f, int64_t B, int64_t TC,
+                                                 int accumulate) {
+  constexpr int VN = Vec16<T>::n;
+  float a[VN];
+#pragma unroll
+  for (int k = 0; k < VN; ++k) a[k] = 0.f;
+  for (int64_t b0 = 0; b0 < B; b0 += 8) {
+    Vec16<T> v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b0 + u < B) v[u] = load16(dout + (b0 + u) * TC + f * VN);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b0 + u < B)
+#pragma unroll
+        for (int k = 0; k < VN; ++k) a[k] += to_acc(v[u].e[k]);
+  }
+  Vec16<T> o;
+  if (accumulate) {
+    const Vec16<T> old = load16(dwpe + f * VN);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(to_acc(old.e[k]) + a[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(a[k]);
+  }
+  store16_stream(dwpe + f * VN, o);
+}
+
+// Launch layout, in block order:
+//   [0, n_tiles)                sort one tile of 1024 keys
+//   + 1                         preset sorted_id to "no id", clear the row bitmap
+//   + pos_blocks                position-table gradient, 1024 vectors per block
+template <typename KeyT, typename IdxT, typename T>
+__global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
     const IdxT *__restrict__ ids, KeyT *__restrict__ tiles, uint32_t *__restrict__ bitmap,
-    int bitmap_words, uint32_t *__restrict__ sorted_id, int64_t n, int n_tiles, int shift,
-    int64_t num_weights, int64_t padding_idx) {
-  __shared__ KeyT keys[kTile];
-  if ((int)blockIdx.x >= n_tiles) {
-    const int64_t t = (int64_t)(blockIdx.x - n_tiles) * kSortThreads + threadIdx.x;
-    const int64_t stride = (int64_t)(gridDim.x - n_tiles) * kSortThreads;
-    for (int64_t i = t; i < bitmap_words; i += stride) bitmap[i] = 0u;
-    for (int64_t i = t; i < n; i += stride) sorted_id[i] = kNoId;
+    int64_t bitmap_words, uint32_t *__restrict__ sorted_id, int64_t n, int n_tiles, int shift,
+    int64_t num_weights, int64_t padding_idx, const T *__restrict__ dout, T *__restrict__ dwpe,
+    int64_t B, int64_t TC, int accumulate) {
+  __shared__ KeyT keys[2][kTile];
+  const int tid = threadIdx.x;
+  const int64_t blk = blockIdx.x;
+  if (blk > n_tiles) {
+    const int64_t f = (blk - n_tiles - 1) * kTile + tid;
+    if (f < TC / Vec16<T>::n) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
     return;
   }
-  const int64_t tile_base = (int64_t)blockIdx.x * kTile;
-  for (int i = threadIdx.x; i < kTile; i += kSortThreads) {
-    const int64_t p = tile_base + i;
-    KeyT key = KeyCodec<KeyT>::kSentinel;
-    if (p < n) {
-      const int64_t id = (int64_t)ids[p];
-      if (id >= 0 && id < num_weights && id != padding_idx)
-        key = KeyCodec<KeyT>::make((uint32_t)id, (uint32_t)p, shift);
-    }
-    keys[i] = key;
+  if (blk == n_tiles) {
+    for (int64_t i = tid; i < bitmap_words; i += kTile) bitmap[i] = 0u;
+    for (int64_t i = tid; i < n; i += kTile) sorted_id[i] = kNoId;
+    return;
   }
-  __syncthreads();
-  // bitonic network, ascending
+  const int64_t p = blk * kTile + tid;
+  KeyT key = KeyCodec<KeyT>::kSentinel;
+  if (p < n) {
+    const int64_t id = (int64_t)ids[p];
+    if (id >= 0 && id < num_weights && id != padding_idx)
+      key = KeyCodec<KeyT>::make((uint32_t)id, (uint32_t)p, shift);
+  }
+  // bitonic network, ascending, one key per lane
+  int buf = 0;
   for (int k = 2; k <= kTile; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
-      const int t = threadIdx.x;
-      const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-      const int partner = i | j;
-      const bool up = (i & k) == 0;
-      const KeyT a = keys[i], b = keys[partner];
-      if ((a > b) == up) {
-        keys[i] = b;
-        keys[partner] = a;
+      KeyT other;
+      if (j >= kWave) {
+        keys[buf][tid] = key;
+        __syncthreads();
+        other = keys[buf][tid ^ j];
+        buf ^= 1;  // the next exchange writes the other array: one barrier per step
+      } else {
+        other = __shfl_xor(key, j, kWave);
       }
-      __syncthreads();
+      const bool up = (tid & k) == 0;     // this 2k-block sorts ascending
+      const bool lower = (tid & j) == 0;  // this lane is the lower index of its pair
+      const KeyT lo = key < other ? key : other;
+      const KeyT hi = key < other ? other : key;
+      key = (lower == up) ? lo : hi;
     }
   }
-  for (int i = threadIdx.x; i < kTile; i += kSortThreads) tiles[tile_base + i] = keys[i];
+  tiles[p] = key;
 }
 
 // One thread per key.  rank = own index in own tile + lower bounds in all
-// other tiles; four tiles are searched side by side so their loads overlap.
-// The global predecessor is the largest of the per-tile predecessors; a key
-// whose predecessor has another id starts a segment.
+// other tiles.  The tiles are staged in LDS a chunk at a time and four of
+// them are searched side by side, so the probes overlap.
+constexpr int kMergeChunkBytes = 32768;
+
 template <typename KeyT>
 __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
     const KeyT *__restrict__ tiles, uint32_t *__restrict__ bitmap,
     uint32_t *__restrict__ sorted_id, uint32_t *__restrict__ sorted_pos, int n_tiles, int shift) {
+  constexpr int kChunkTiles = kMergeChunkBytes / (kTile * (int)sizeof(KeyT));
   constexpr int kSide = 4;
+  constexpr int kVecPerThread = kMergeChunkBytes / 16 / kThreads;  // 8
+  __shared__ u32x4 staged_raw[kMergeChunkBytes / 16];
+  const KeyT *staged = reinterpret_cast<const KeyT *>(staged_raw);
   const int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  const int own = (int)(g / kTile);
+  const int own = (int)(g / kTile);  // block-uniform: 256 divides 1024
   const int local = (int)(g % kTile);
-  if (own >= n_tiles) return;
   const KeyT key = tiles[g];
-  if (key == KeyCodec<KeyT>::kSentinel) return;
+  const bool real = key != KeyCodec<KeyT>::kSentinel;
   int64_t rank = local;
+  // the global predecessor is the largest of the per-tile predecessors
   bool has_pred = local > 0;
   KeyT pred = has_pred ? tiles[g - 1] : (KeyT)0;
-  for (int b0 = 0; b0 < n_tiles; b0 += kSide) {
-    const KeyT *tile[kSide];
-    int lb[kSide];
+  for (int c0 = 0; c0 < n_tiles; c0 += kChunkTiles) {
+    const int c_tiles = n_tiles - c0 < kChunkTiles ? n_tiles - c0 : kChunkTiles;
+    const int c_vecs = c_tiles * kTile * (int)sizeof(KeyT) / 16;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(tiles + (int64_t)c0 * kTile);
+    u32x4 v[kVecPerThread];
 #pragma unroll
-    for (int u = 0; u < kSide; ++u) {
-      const int b = b0 + u < n_tiles ? b0 + u : n_tiles - 1;
-      tile[u] = tiles + (int64_t)b * kTile;
-      lb[u] = 0;
+    for (int u = 0; u < kVecPerThread; ++u) {
+      const int i = u * kThreads + threadIdx.x;
+      if (i < c_vecs) v[u] = src[i];
     }
-    // lower bound in a power-of-two tile: kTile/2, kTile/4, ... 1, then one last probe
-    for (int step = kTile >> 1; step > 0; step >>= 1) {
-      KeyT probe[kSide];
+    __syncthreads();  // the previous chunk is no longer being searched
 #pragma unroll
-      for (int u = 0; u < kSide; ++u) probe[u] = tile[u][lb[u] + step - 1];
-#pragma unroll
-      for (int u = 0; u < kSide; ++u) lb[u] += probe[u] < key ? step : 0;
+    for (int u = 0; u < kVecPerThread; ++u) {
+      const int i = u * kThreads + threadIdx.x;
+      if (i < c_vecs) staged_raw[i] = v[u];
     }
-    KeyT last[kSide], before[kSide];
+    __syncthreads();
+    for (int b0 = 0; b0 < c_tiles; b0 += kSide) {
+      const KeyT *tile[kSide];
+      int lb[kSide];
 #pragma unroll
-    for (int u = 0; u < kSide; ++u) {
-      last[u] = tile[u][lb[u]];
-      before[u] = lb[u] > 0 ? tile[u][lb[u] - 1] : (KeyT)0;
-    }
-#pragma unroll
-    for (int u = 0; u < kSide; ++u) {
-      const int b = b0 + u;
-      if (b >= n_tiles || b == own) continue;
-      // lb is the count of keys < key; the key just below it is the tile's predecessor
-      KeyT cand = before[u];
-      int count = lb[u];
-      if (last[u] < key) {
-        cand = last[u];
-        count += 1;
+      for (int u = 0; u < kSide; ++u) {
+        const int b = b0 + u < c_tiles ? b0 + u : c_tiles - 1;
+        tile[u] = staged + b * kTile;
+        lb[u] = 0;
       }
-      rank += count;
-      if (count > 0 && (!has_pred || cand > pred)) {
-        pred = cand;
-        has_pred = true;
+      // lower bound in a power-of-two tile: kTile/2, kTile/4, ... 1, then one last probe
+      for (int step = kTile >> 1; step > 0; step >>= 1) {
+        KeyT probe[kSide];
+#pragma unroll
+        for (int u = 0; u < kSide; ++u) probe[u] = tile[u][lb[u] + step - 1];
+#pragma unroll
+        for (int u = 0; u < kSide; ++u) lb[u] += probe[u] < key ? step : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kSide; ++u) {
+        const int b = c0 + b0 + u;
+        if (b0 + u >= c_tiles || b == own) continue;
+        // lb counts the keys < key so far; the key just below the bound is the tile's predecessor
+        const KeyT at = tile[u][lb[u]];
+        const int count = lb[u] + (at < key ? 1 : 0);
+        rank += count;
+        if (count > 0) {
+          const KeyT cand = tile[u][count - 1];
+          if (!has_pred || cand > pred) pred = cand;
+          has_pred = true;
+        }
       }
     }
   }
+  if (!real) return;
   const uint32_t id = KeyCodec<KeyT>::id(key, shift);
   sorted_id[rank] = id;
   sorted_pos[rank] = KeyCodec<KeyT>::pos(key, shift);
+  // the first key of an id marks the row as touched
   if (!has_pred || KeyCodec<KeyT>::id(pred, shift) != id) atomicOr(&bitmap[id >> 5], 1u << (id & 31));
 }
 
 // ------------------------------------------------------ backward: reduction
-constexpr int kWin = 8;  // sorted entries per wavefront window
-constexpr int kVpl = 2;  // 16-byte column vectors per lane per column chunk
+constexpr int kRedThreads = 1024;
+constexpr int kRedWaves = kRedThreads / kWave;  // 16
+constexpr int kOwn = kWindow / kRedWaves;       // 4 sorted entries per wave
+constexpr int kVpl = 2;                         // 16-byte column vectors per lane per column chunk
 
-template <typename T>
-struct Row2 {
-  Vec16<T> v[kVpl];
-};
+// Workgroup w reduces sorted entries [64 w, 64 w + 64).  partial rows live at
+// partial[(w*2 + slot) * C]: slot 0 for a run that came in over the window's
+// left edge and ends inside, slot 1 for a run that leaves over its right edge.
+constexpr int kFillRows = 64;  // rows per zero-fill workgroup
 
-// Window w covers sorted entries [8w, 8w+8).  partial rows live at
-// partial[(w*2 + slot) * C]: slot 1 for the run that contains the window's
-// last entry, slot 0 for a cut run that contains only its first.
+// Launch layout: [0, n_windows) reduce one window each; the rest zero 64 rows each.
 template <typename T>
-__global__ __launch_bounds__(kThreads) void emb_bwd_window_kernel(
+__global__ __launch_bounds__(kRedThreads) void emb_bwd_reduce_kernel(
     const T *__restrict__ dout, const uint32_t *__restrict__ sorted_id,
-    const uint32_t *__restrict__ sorted_pos, T *__restrict__ dweight, float *__restrict__ partial,
-    int64_t n, int64_t C, int accumulate) {
+    const uint32_t *__restrict__ sorted_pos, const uint32_t *__restrict__ bitmap,
+    T *__restrict__ dweight, float *__restrict__ partial, int64_t n, int64_t C,
+    int64_t num_weights, int64_t n_windows, int accumulate) {
   constexpr int VN = Vec16<T>::n;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t w = (int64_t)blockIdx.x * (kThreads / kWave) + (threadIdx.x >> 6);
-  const int64_t p0 = w * kWin;
-  if (p0 >= n) return;  // wave-uniform
-  // ids of entries p0-1 .. p0+8 (kNoId outside [0,n) and for unused slots)
-  uint32_t id[kWin + 2], pos[kWin];
-#pragma unroll
-  for (int e = -1; e <= kWin; ++e) {
-    const int64_t p = p0 + e;
-    id[e + 1] = (p >= 0 && p < n) ? sorted_id[p] : kNoId;
-  }
-  if (id[1] == kNoId) return;  // nothing valid in this window
-#pragma unroll
-  for (int e = 0; e < kWin; ++e) pos[e] = id[e + 1] != kNoId ? sorted_pos[p0 + e] : 0u;
-
+  constexpr int kChunkCols = kWave * kVpl * VN;
+  extern __shared__ float lds[];  // [16 waves][2 slots][kChunkCols]
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
   const int nvec = (int)(C / VN);
+  if ((int64_t)blockIdx.x >= n_windows) {
+    // ---- zero fill of rows nobody indexed; wave w takes rows w, w + 16, ... of this block's 64
+    const int64_t row0 = ((int64_t)blockIdx.x - n_windows) * kFillRows;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int r = 0; r < kFillRows / kRedWaves; ++r) {
+      const int64_t row = row0 + wave + (int64_t)r * kRedWaves;
+      if (row >= num_weights) break;
+      if ((bitmap[row >> 5] >> (row & 31)) & 1u) continue;  // wave-uniform
+      u32x4 *dst = reinterpret_cast<u32x4 *>(dweight + row * C);
+      for (int idx = lane; idx < nvec; idx += kWave) __builtin_nontemporal_store(z, dst + idx);
+    }
+    return;
+  }
+  const int64_t w = blockIdx.x;
+  const int64_t p0 = w * kWindow;
+
+  // ---- ids of the window (lane l <-> entry p0 + l), the entry before and the entry after
+  const int64_t p = p0 + lane;
+  const uint32_t my_id = p < n ? sorted_id[p] : kNoId;
+  const uint32_t prev_id = (p > 0 && p <= n) ? sorted_id[p - 1] : kNoId;
+  const uint64_t valid = __ballot(my_id != kNoId);
+  if (valid == 0) return;  // nothing sorted into this window
+  const int n_valid = __popcll(valid);  // valid entries are a prefix of the window
+  // true segment heads, and run starts inside the window (a head, or entry 0)
+  const uint64_t heads = __ballot(my_id != kNoId && (p == 0 || my_id != prev_id));
+  const uint64_t starts = heads | 1ull;
+  const uint32_t next_id = (p0 + kWindow < n) ? sorted_id[p0 + kWindow] : kNoId;  // uniform load
+  const uint32_t last_id = __shfl(my_id, n_valid - 1, kWave);
+  const bool leaves = n_valid == kWindow && next_id == last_id;    // last run goes over the right edge
+
+  // Of a run [a, b) inside the window: is it a whole segment?
+  //   begins here  <=> a is a true head          ends here <=> b < n_valid, or b == n_valid and !leaves
+  auto run_end = [&](int a) -> int {  // end of the run that starts at entry a
+    const uint64_t later = a >= 63 ? 0ull : (starts >> (a + 1)) << (a + 1);
+    const int b = later ? __ffsll((long long)later) - 1 : n_valid;
+    return b < n_valid ? b : n_valid;
+  };
+
   for (int cb = 0; cb < nvec; cb += kWave * kVpl) {
-    Row2<T> r[kWin];
+    // ---- level 1: this wave's four entries
+    const int e0 = wave * kOwn;
+    Vec16<T> r[kOwn][kVpl];
+    // lanes 0..3 fetch the four positions together; the rows are then loaded at once
+    const uint32_t lane_pos = (lane < kOwn && e0 + lane < n_valid) ? sorted_pos[p0 + e0 + lane] : 0u;
 #pragma unroll
-    for (int e = 0; e < kWin; ++e) {
+    for (int e = 0; e < kOwn; ++e) {
+      if (e0 + e < n_valid) {
+        const int64_t pos = __shfl(lane_pos, e, kWave);
 #pragma unroll
-      for (int j = 0; j < kVpl; ++j) {
-        const int idx = cb + lane + kWave * j;
-        if (id[e + 1] != kNoId && idx < nvec) {
-          r[e].v[j] = load16_stream(dout + (int64_t)pos[e] * C + (int64_t)idx * VN);
+        for (int j = 0; j < kVpl; ++j) {
+          const int idx = cb + lane + kWave * j;
+          if (idx < nvec) r[e][j] = load16_stream(dout + pos * C + (int64_t)idx * VN);
         }
       }
     }
     float acc[kVpl][VN];
-    int run_start = 0;
+    int piece_start = e0;
 #pragma unroll
-    for (int e = 0; e < kWin; ++e) {
-      if (id[e + 1] == kNoId) break;
-      if (e == 0 || id[e + 1] != id[e]) {
-        run_start = e;
+    for (int e = 0; e < kOwn; ++e) {
+      const int q = e0 + e;
+      if (q >= n_valid) break;
+      const bool starts_here = (starts >> q) & 1ull;
+      if (e == 0 || starts_here) {
+        piece_start = q;
 #pragma unroll
         for (int j = 0; j < kVpl; ++j)
 #pragma unroll
@@ -311,16 +406,21 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_window_kernel(
       for (int j = 0; j < kVpl; ++j) {
         if (cb + lane + kWave * j < nvec) {
 #pragma unroll
-          for (int k = 0; k < VN; ++k) acc[j][k] += to_acc(r[e].v[j].e[k]);
+          for (int k = 0; k < VN; ++k) acc[j][k] += to_acc(r[e][j].e[k]);
         }
       }
-      const bool run_ends = e == kWin - 1 || id[e + 2] != id[e + 1];
-      if (run_ends) {
-        // does the segment start / end inside this window?
-        const bool seg_begins = run_start > 0 || id[0] != id[e + 1];
-        const bool seg_ends = id[e + 2] != id[e + 1];
+      const bool piece_ends = e == kOwn - 1 || q + 1 >= n_valid || ((starts >> (q + 1)) & 1ull);
+      if (!piece_ends) continue;
+      // the run this piece belongs to
+      const bool run_starts_in_piece = (starts >> piece_start) & 1ull;
+      const bool run_ends_in_piece = q + 1 >= n_valid || ((starts >> (q + 1)) & 1ull);
+      const uint32_t id = __shfl(my_id, q, kWave);
+      if (run_starts_in_piece && run_ends_in_piece) {
+        // a whole run of the window, inside one wave
+        const bool seg_begins = (heads >> piece_start) & 1ull;
+        const bool seg_ends = !(q + 1 >= n_valid && leaves);
         if (seg_begins && seg_ends) {
-          T *dst = dweight + (int64_t)id[e + 1] * C;
+          T *dst = dweight + (int64_t)id * C;
 #pragma unroll
           for (int j = 0; j < kVpl; ++j) {
             const int idx = cb + lane + kWave * j;
@@ -338,155 +438,127 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_window_kernel(
             }
           }
         } else {
-          const int slot = e == kWin - 1 ? 1 : 0;
-          float *dst = partial + (w * 2 + slot) * C;
+          float *dst = partial + (w * 2 + (seg_ends ? 0 : 1)) * C;
 #pragma unroll
           for (int j = 0; j < kVpl; ++j) {
             const int idx = cb + lane + kWave * j;
             if (idx < nvec) {
 #pragma unroll
-              for (int q = 0; q < VN / 4; ++q) {
-                Vec16<float> o;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) o.e[k] = acc[j][q * 4 + k];
-                store16(dst + (int64_t)idx * VN + q * 4, o);
-              }
+              for (int k = 0; k < VN; ++k) dst[(int64_t)idx * VN + k] = acc[j][k];
             }
+          }
+        }
+      } else {
+        // part of a run that spans waves: slot 1 if it reaches this wave's last entry
+        const int slot = e == kOwn - 1 ? 1 : 0;
+        float *dst = lds + (wave * 2 + slot) * kChunkCols;
+#pragma unroll
+        for (int j = 0; j < kVpl; ++j)
+#pragma unroll
+          for (int k = 0; k < VN; ++k) dst[(lane + kWave * j) * VN + k] = acc[j][k];
+      }
+    }
+    __syncthreads();
+    // ---- level 2: runs of the window that span waves, folded in wave order
+    {
+      // a run spans waves exactly when some wave's first entry (4, 8, ... 60) is valid and is
+      // not a run start; walk those entries and fold each run once
+      uint64_t cont = ~starts & valid & 0x1111111111111110ull;
+      int prev_a = -1;
+      while (cont) {
+        const int q = __ffsll((long long)cont) - 1;
+        cont &= cont - 1;
+        const int a = 63 - __clzll((long long)(starts & ((1ull << q) - 1ull)));  // its run's start
+        if (a == prev_a) continue;
+        prev_a = a;
+        const int b = run_end(a);
+        const int wa = a / kOwn, wb = (b - 1) / kOwn;
+        const int c = tid;       // one column of the chunk per thread
+        const int64_t col = (int64_t)cb * VN + c;
+        // read the id while every lane is still active: a shuffle cannot read an idle lane
+        const uint32_t id = __shfl(my_id, a, kWave);
+        if (c < kChunkCols && col < C) {
+          float t = 0.f;
+          for (int ww = wa; ww <= wb; ++ww) {
+            // wave ww's piece of this run reaches its last entry unless the run ends inside it
+            const int slot = (ww < wb || (b % kOwn) == 0) ? 1 : 0;
+            t += lds[(ww * 2 + slot) * kChunkCols + c];
+          }
+          const bool seg_begins = (heads >> a) & 1ull;
+          const bool seg_ends = !(b >= n_valid && leaves);
+          if (seg_begins && seg_ends) {
+            T *dst = dweight + (int64_t)id * C;
+            if (accumulate) t += to_acc(dst[col]);
+            dst[col] = from_acc<T>(t);
+          } else {
+            partial[(w * 2 + (seg_ends ? 0 : 1)) * C + col] = t;
           }
         }
       }
     }
+    __syncthreads();
   }
+
 }
 
-constexpr int kFinThreads = 1024;
-constexpr int kFinGroups = 4;  // partial rows are dealt to 4 thread groups
-
-// Launch layout of the finish kernel, in block order:
-//   [0, n_windows)                       : long-segment fix-up, one block per window
-//   [n_windows, n_windows + pos_blocks)  : position table gradient
-//   the rest                             : zero fill of rows never indexed
+// The last level of the segmented sum.  Workgroup w looks at window w: if the
+// run that leaves it over the right edge began in it (a true segment head),
+// this is that segment's first window, and the workgroup adds the segment's
+// partial rows in window order: slot 1 of every window the segment leaves,
+// slot 0 of the one it ends in.
 template <typename T>
-__global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
-    const T *__restrict__ dout, const uint32_t *__restrict__ sorted_id,
-    const uint32_t *__restrict__ bitmap, const float *__restrict__ partial,
-    T *__restrict__ dweight, T *__restrict__ dwpe, int64_t n, int64_t C, int64_t num_weights,
-    int64_t B, int64_t T_len, int64_t n_windows, int64_t pos_blocks, int accumulate,
-    int do_fill) {
-  constexpr int VN = Vec16<T>::n;
-  extern __shared__ float lds[];  // [kFinGroups][256 * 4] column chunk
-  const int64_t blk = blockIdx.x;
-  if (blk < n_windows) {
-    // ---- fix-up: only a window whose last run starts a segment that runs on
-    const int64_t w = blk;
-    const int64_t first = w * kWin;
-    const int64_t last = first + kWin - 1;
-    if (last + 1 >= n) return;
-    const uint32_t id = sorted_id[last];
-    if (id == kNoId || sorted_id[last + 1] != id) return;  // segment ends in this window
-    // does the segment start in this window?  (entries are sorted, so "the
-    // entry before the window has this id" means it started earlier)
-    if (first > 0 && sorted_id[first - 1] == id) return;
-    // first entry after `last` that has another id, found 1024 entries at a time
-    __shared__ int64_t seg_end_sh;
-    int64_t seg_end = n;
-    for (int64_t base = last + 1; base < n; base += kFinThreads) {
-      const int64_t p = base + threadIdx.x;
-      const bool differs = p < n && sorted_id[p] != id;
-      if (threadIdx.x == 0) seg_end_sh = n;
-      __syncthreads();
-      if (differs) atomicMin((unsigned long long *)&seg_end_sh, (unsigned long long)p);
-      __syncthreads();
-      seg_end = seg_end_sh;
-      __syncthreads();
-      if (seg_end < n) break;
-    }
-    const int64_t after = seg_end - (last + 1);  // entries of the segment past this window
-    const int64_t full = after / kWin;           // windows it covers completely
-    const bool head_cut = after % kWin != 0;     // then a cut run in the next one
-    // partial rows to add, in window order: (w,1), (w+1,1) ... (w+full,1), then (w+full+1,0)
-    const int64_t n_parts = 1 + full + (head_cut ? 1 : 0);
-    const int group = threadIdx.x >> 8;   // 0..3
-    const int lane256 = threadIdx.x & 255;
-    const int64_t c4 = C / 4;             // float4 columns
-    T *dst = dweight + (int64_t)id * C;
-    for (int64_t cb = 0; cb < c4; cb += 256) {
-      const int64_t col4 = cb + lane256;
-      float a[4] = {0.f, 0.f, 0.f, 0.f};
-      if (col4 < c4) {
-        for (int64_t i = group; i < n_parts; i += kFinGroups) {
-          const int64_t win = w + i;
-          const int slot = (head_cut && i == n_parts - 1) ? 0 : 1;
-          const Vec16<float> v = load16(partial + (win * 2 + slot) * C + col4 * 4);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) a[k] += v.e[k];
-        }
+__global__ __launch_bounds__(kRedThreads) void emb_bwd_finish_kernel(
+    const uint32_t *__restrict__ sorted_id, const float *__restrict__ partial,
+    T *__restrict__ dweight, int64_t n, int64_t C, int accumulate) {
+  __shared__ int first_other[kRedWaves];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int64_t w = blockIdx.x;
+  const int64_t last = w * kWindow + kWindow - 1;
+  if (last + 1 >= n) return;  // nothing after this window
+  const uint32_t id = sorted_id[last];
+  if (id == kNoId || sorted_id[last + 1] != id) return;  // no run leaves this window
+  // its run began in this window unless the whole window (and the entry before it) has this id
+  if (sorted_id[w * kWindow] == id && w > 0 && sorted_id[w * kWindow - 1] == id) return;
+  // windows after w whose last entry still has this id are left by the segment too; lane t
+  // probes window w + 1 + t, 1024 windows per round
+  int64_t w_hi = -1;  // the window the segment ends in
+  for (int64_t base = w + 1; w_hi < 0; base += kRedThreads) {
+    const int64_t ww = base + tid;
+    const int64_t q = ww * kWindow + kWindow - 1;
+    const bool other = q >= n || sorted_id[q] != id;
+    const uint64_t m = __ballot(other);
+    if (lane == 0) first_other[wave] = m ? __ffsll((long long)m) - 1 : -1;
+    __syncthreads();
+    for (int k = 0; k < kRedWaves; ++k) {
+      if (first_other[k] >= 0) {
+        w_hi = base + k * kWave + first_other[k];
+        break;
       }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) lds[(group * 256 + lane256) * 4 + k] = a[k];
-      __syncthreads();
-      if (group == 0 && col4 < c4) {
-        float t[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          t[k] = lds[(0 * 256 + lane256) * 4 + k];
-#pragma unroll
-          for (int g2 = 1; g2 < kFinGroups; ++g2) t[k] += lds[(g2 * 256 + lane256) * 4 + k];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int64_t c = col4 * 4 + k;
-          const float old = accumulate ? to_acc(dst[c]) : 0.f;
-          dst[c] = from_acc<T>(old + t[k]);
-        }
-      }
-      __syncthreads();
     }
-    return;
+    __syncthreads();
   }
-  const int nvec = (int)(C / VN);
-  if (blk < n_windows + pos_blocks) {
-    // ---- dwpe[t, :] (+)= sum_b dout[b, t, :], ascending b
-    const int64_t f = (blk - n_windows) * kFinThreads + threadIdx.x;
-    if (f >= T_len * nvec) return;
-    float a[VN];
-#pragma unroll
-    for (int k = 0; k < VN; ++k) a[k] = 0.f;
-#pragma unroll 8
-    for (int64_t b = 0; b < B; ++b) {
-      const Vec16<T> v = load16(dout + b * T_len * C + f * VN);
-#pragma unroll
-      for (int k = 0; k < VN; ++k) a[k] += to_acc(v.e[k]);
+  // w_hi is the first window whose last entry is not this id.  The segment ends inside it when
+  // its first entry still has the id, otherwise exactly at the end of the window before.
+  const bool tail = w_hi * kWindow < n && sorted_id[w_hi * kWindow] == id;
+  const int64_t w_end = tail ? w_hi : w_hi - 1;  // the window the segment ends in (> w)
+  T *dst = dweight + (int64_t)id * C;
+  for (int64_t col = tid; col < C; col += kRedThreads) {
+    float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+    int64_t ww = w;
+    // every window before the last is left over its right edge (slot 1)
+    for (; ww + 4 <= w_end; ww += 4) {
+      t0 += partial[((ww + 0) * 2 + 1) * C + col];
+      t1 += partial[((ww + 1) * 2 + 1) * C + col];
+      t2 += partial[((ww + 2) * 2 + 1) * C + col];
+      t3 += partial[((ww + 3) * 2 + 1) * C + col];
     }
-    Vec16<T> o;
-    if (accumulate) {
-      const Vec16<T> old = load16(dwpe + f * VN);
-#pragma unroll
-      for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(to_acc(old.e[k]) + a[k]);
-    } else {
-#pragma unroll
-      for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(a[k]);
-    }
-    store16_stream(dwpe + f * VN, o);
-    return;
-  }
-  if (!do_fill) return;
-  // ---- zero fill: 4 vectors per thread
-  const int64_t chunk_base = (blk - n_windows - pos_blocks) * (kFinThreads * 4);
-  const int64_t row_base = chunk_base / nvec;
-  const uint32_t rem_base = (uint32_t)(chunk_base - row_base * nvec);
-  const int64_t total = num_weights * nvec;
-  Vec16<T> z;
-#pragma unroll
-  for (int k = 0; k < VN; ++k) z.e[k] = T{};
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int64_t f = chunk_base + (int64_t)u * kFinThreads + threadIdx.x;
-    if (f < total) {
-      const uint32_t local = rem_base + (uint32_t)(u * kFinThreads) + threadIdx.x;
-      const int64_t row = row_base + local / (uint32_t)nvec;
-      if (((bitmap[row >> 5] >> (row & 31)) & 1u) == 0u) store16_stream(dweight + f * VN, z);
-    }
+    for (; ww < w_end; ++ww) t0 += partial[(ww * 2 + 1) * C + col];
+    t1 += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
+    float t = (t0 + t1) + (t2 + t3);
+    if (accumulate) t += to_acc(dst[col]);
+    dst[col] = from_acc<T>(t);
   }
 }
 
@@ -538,8 +610,8 @@ struct BwdLayout {
   int shift = 0;
   bool key64 = false;
   int64_t n_tiles = 0;
-  int64_t bitmap_words = 0;
   int64_t n_windows = 0;
+  int64_t bitmap_words = 0;
   size_t off_bitmap = 0, off_tiles = 0, off_sorted_id = 0, off_sorted_pos = 0, off_partial = 0;
   size_t bytes = 0;
 };
@@ -553,8 +625,8 @@ BwdLayout bwd_layout(int64_t n, int64_t C, int64_t num_weights) {
   while ((1ll << L.shift) < padded) ++L.shift;
   // ((V-1) << shift) | (2^shift - 1) must stay below the 32-bit sentinel
   L.key64 = L.shift >= 32 || ((uint64_t)num_weights << L.shift) > 0xFFFFFFFFull;
+  L.n_windows = ceil_div(n, (int64_t)kWindow);
   L.bitmap_words = ceil_div(num_weights, (int64_t)32);
-  L.n_windows = ceil_div(n, (int64_t)kWin);
   size_t o = 0;
   L.off_bitmap = o;
   o = align256(o + (size_t)L.bitmap_words * 4);
@@ -617,7 +689,6 @@ int fwd_dispatch(const void *weight, const void *wpe, const void *ids, void *out
       !aligned_to(ids, idx_dtype == CS_I64 ? 8 : 4))
     return CS_ERR_MISALIGNED;
   hipStream_t s = as_stream(stream);
-  // a plain gather is a byte copy: 16-bit types share one kernel
   switch (dtype) {
     case CS_F32:
       return fwd_idx<float, ADD>(weight, wpe, ids, out, n_rows, C, num_weights, T_len, idx_dtype, s);
@@ -631,76 +702,97 @@ int fwd_dispatch(const void *weight, const void *wpe, const void *ids, void *out
   return CS_ERR_UNSUPPORTED;
 }
 
-template <typename KeyT, typename IdxT>
+// Sort + merge.  The sort launch also sums dwpe (`fused_positions`) on the CUs the sort
+// leaves idle.
+template <typename KeyT, typename IdxT, typename T>
 int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_t num_weights,
-                int64_t padding_idx, hipStream_t s) {
+                int64_t padding_idx, const T *dout, T *dwpe, bool fused_positions, int64_t B,
+                int64_t TC, int accumulate, hipStream_t s) {
   KeyT *tiles = reinterpret_cast<KeyT *>(ws + L.off_tiles);
   uint32_t *bitmap = reinterpret_cast<uint32_t *>(ws + L.off_bitmap);
   uint32_t *sorted_id = reinterpret_cast<uint32_t *>(ws + L.off_sorted_id);
   uint32_t *sorted_pos = reinterpret_cast<uint32_t *>(ws + L.off_sorted_pos);
-  const int extra = 8;  // blocks that clear the bitmap and preset sorted_id
-  emb_bwd_tile_sort_kernel<KeyT, IdxT>
-      <<<dim3((unsigned)(L.n_tiles + extra)), dim3(kSortThreads), 0, s>>>(
-          (const IdxT *)ids, tiles, bitmap, (int)L.bitmap_words, sorted_id, n, (int)L.n_tiles,
-          L.shift, num_weights, padding_idx);
+  const int64_t pos_blocks = fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)kTile) : 0;
+  const int64_t blocks = L.n_tiles + 1 + pos_blocks;
+  if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  emb_bwd_tile_sort_kernel<KeyT, IdxT, T><<<dim3((unsigned)blocks), dim3(kTile), 0, s>>>(
+      (const IdxT *)ids, tiles, bitmap, L.bitmap_words, sorted_id, n, (int)L.n_tiles, L.shift,
+      num_weights, padding_idx, dout, dwpe, B, TC, accumulate);
   int st = launch_status();
   if (st != CS_OK) return st;
-  const int64_t blocks = ceil_div(L.n_tiles * kTile, (int64_t)kThreads);
-  emb_bwd_merge_kernel<KeyT><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+  const int64_t mblocks = L.n_tiles * kTile / kThreads;
+  emb_bwd_merge_kernel<KeyT><<<dim3((unsigned)mblocks), dim3(kThreads), 0, s>>>(
       tiles, bitmap, sorted_id, sorted_pos, (int)L.n_tiles, L.shift);
   return launch_status();
+}
+
+// The reduce kernel asks for 128 KB of LDS, above the 64 KB a launch gets by default.
+template <typename T>
+int allow_reduce_lds(size_t bytes) {
+  static bool done[64] = {false};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  if (!done[dev]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&emb_bwd_reduce_kernel<T>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+    done[dev] = true;
+  }
+  return CS_OK;
 }
 
 template <typename T>
 int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char *ws,
               const BwdLayout &L, int64_t n, int64_t C, int64_t num_weights, int64_t padding_idx,
               int64_t B, int64_t T_len, int idx_dtype, int accumulate, hipStream_t s) {
+  constexpr int VN = Vec16<T>::n;
+  const bool vec_ok = !std::is_same_v<T, double> && C % VN == 0 && is_aligned16(dout) &&
+                      is_aligned16(dweight) && (!dwpe || is_aligned16(dwpe));
+  const bool fused_positions = vec_ok && dwpe != nullptr;
+  const int64_t TC = T_len * C;
   int st;
+#define CS_SORT(KeyT, IdxT)                                                                      \
+  sort_launch<KeyT, IdxT, T>(ids, ws, L, n, num_weights, padding_idx, (const T *)dout, (T *)dwpe, \
+                             fused_positions, B, TC, accumulate, s)
   if (L.key64) {
-    st = idx_dtype == CS_I64
-             ? sort_launch<uint64_t, int64_t>(ids, ws, L, n, num_weights, padding_idx, s)
-             : sort_launch<uint64_t, int32_t>(ids, ws, L, n, num_weights, padding_idx, s);
+    st = idx_dtype == CS_I64 ? CS_SORT(uint64_t, int64_t) : CS_SORT(uint64_t, int32_t);
   } else {
-    st = idx_dtype == CS_I64
-             ? sort_launch<uint32_t, int64_t>(ids, ws, L, n, num_weights, padding_idx, s)
-             : sort_launch<uint32_t, int32_t>(ids, ws, L, n, num_weights, padding_idx, s);
+    st = idx_dtype == CS_I64 ? CS_SORT(uint32_t, int64_t) : CS_SORT(uint32_t, int32_t);
   }
+#undef CS_SORT
   if (st != CS_OK) return st;
   const uint32_t *bitmap = reinterpret_cast<const uint32_t *>(ws + L.off_bitmap);
   const uint32_t *sorted_id = reinterpret_cast<const uint32_t *>(ws + L.off_sorted_id);
   const uint32_t *sorted_pos = reinterpret_cast<const uint32_t *>(ws + L.off_sorted_pos);
-  float *partial = reinterpret_cast<float *>(ws + L.off_partial);
-  constexpr int VN = Vec16<T>::n;
-  const bool vec_ok = !std::is_same_v<T, double> && C % VN == 0 && C % 4 == 0 &&
-                      is_aligned16(dout) && is_aligned16(dweight) && (!dwpe || is_aligned16(dwpe));
   if (!vec_ok) {
     if (num_weights > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
     emb_bwd_rows_general_kernel<T><<<dim3((unsigned)num_weights), dim3(kThreads), 0, s>>>(
         (const T *)dout, sorted_id, sorted_pos, (T *)dweight, n, C, accumulate);
     st = launch_status();
     if (st != CS_OK || !dwpe) return st;
-    int64_t blocks = ceil_div(T_len * C, (int64_t)kThreads);
+    int64_t blocks = ceil_div(TC, (int64_t)kThreads);
     if (blocks > 65536) blocks = 65536;
     emb_bwd_positions_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-        (const T *)dout, (T *)dwpe, B, T_len * C, accumulate);
+        (const T *)dout, (T *)dwpe, B, TC, accumulate);
     return launch_status();
   }
   if constexpr (!std::is_same_v<T, double>) {
-    const int64_t win_blocks = ceil_div(L.n_windows, (int64_t)(kThreads / kWave));
-    emb_bwd_window_kernel<T><<<dim3((unsigned)win_blocks), dim3(kThreads), 0, s>>>(
-        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, partial, n, C, accumulate);
-    st = launch_status();
-    if (st != CS_OK) return st;
-    const int64_t nvec = C / VN;
-    const int64_t pos_blocks = dwpe ? ceil_div(T_len * nvec, (int64_t)kFinThreads) : 0;
-    const int64_t fill_blocks =
-        accumulate ? 0 : ceil_div(num_weights * nvec, (int64_t)kFinThreads * 4);
-    const int64_t blocks = L.n_windows + pos_blocks + fill_blocks;
+    float *partial = reinterpret_cast<float *>(ws + L.off_partial);
+    const int64_t windows = n > 0 ? L.n_windows : 0;
+    const int64_t fill_blocks = accumulate ? 0 : ceil_div(num_weights, (int64_t)kFillRows);
+    const int64_t blocks = windows + fill_blocks;
     if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
-    const size_t lds = (size_t)kFinGroups * 256 * 4 * sizeof(float);
-    emb_bwd_finish_kernel<T><<<dim3((unsigned)blocks), dim3(kFinThreads), lds, s>>>(
-        (const T *)dout, sorted_id, bitmap, partial, (T *)dweight, (T *)dwpe, n, C, num_weights, B,
-        T_len, L.n_windows, pos_blocks, accumulate, accumulate ? 0 : 1);
+    if (blocks == 0) return CS_OK;
+    const size_t lds = (size_t)kRedWaves * 2 * kWave * kVpl * VN * sizeof(float);
+    st = allow_reduce_lds<T>(lds);
+    if (st != CS_OK) return st;
+    emb_bwd_reduce_kernel<T><<<dim3((unsigned)blocks), dim3(kRedThreads), lds, s>>>(
+        (const T *)dout, sorted_id, sorted_pos, bitmap, (T *)dweight, partial, n, C, num_weights,
+        windows, accumulate);
+    st = launch_status();
+    if (st != CS_OK || windows == 0) return st;
+    emb_bwd_finish_kernel<T><<<dim3((unsigned)windows), dim3(kRedThreads), 0, s>>>(
+        sorted_id, partial, (T *)dweight, n, C, accumulate);
     return launch_status();
   }
   return CS_ERR_UNSUPPORTED;

@@ -85,7 +85,34 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 constexpr int kLnThreads = 256;  // 4 waves
 
 // ------------------------------------------------------------ fast forward
-// VPL: 16-byte x vectors per lane; R: rows per wave.
+// VPL: 16-byte x vectors per lane; R: rows a wave handles per step.  A wave
+// keeps gamma and beta for its columns in registers and walks rows
+// gw*R, (gw + n_waves)*R, ...; the next step's rows are loaded before the
+// current ones are normalised, so loads overlap the arithmetic and the
+// parameters are read once per wave, not once per row.
+// VN is the column count per vector position (set by x's type); T may be wider.
+template <typename T, int VN, int VPL, int R>
+struct RowSet {
+  Raw<T, VN> v[R][VPL];
+};
+
+template <typename T, int VN, int VPL, int R>
+__device__ __forceinline__ void load_rows(RowSet<T, VN, VPL, R> &dst, const T *__restrict__ src,
+                                          int64_t row0, int64_t rows, int C, int nvec, int lane) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int idx = lane + kWave * j;
+      if (idx < nvec && row0 + r < rows) {
+        dst.v[r][j] = load_raw<T, VN>(src + (row0 + r) * C + (int64_t)idx * VN);
+      } else {
+        dst.v[r][j] = zero_raw<T, VN>();
+      }
+    }
+  }
+}
+
 template <typename TX, typename TY, typename TP, int VPL, int R>
 __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
     const TX *__restrict__ x, const TP *__restrict__ gamma, const TP *__restrict__ beta,
@@ -94,85 +121,86 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   constexpr int VN = Vec16<TX>::n;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t gw = (int64_t)blockIdx.x * (kLnThreads / kWave) + (threadIdx.x >> 6);
-  const int64_t row0 = gw * R;
-  if (row0 >= rows) return;  // wave-uniform
+  const int64_t step = (int64_t)gridDim.x * (kLnThreads / kWave) * R;
   const int nvec = C / VN;
+  int64_t row0 = gw * R;
+  if (row0 >= rows) return;  // wave-uniform
 
-  Raw<TX, VN> xr[R][VPL];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      const int idx = lane + kWave * j;
-      if (idx < nvec && row0 + r < rows) {
-        xr[r][j] = load_raw<TX, VN>(x + (row0 + r) * C + (int64_t)idx * VN);
-      } else {
-        xr[r][j] = zero_raw<TX, VN>();
-      }
-    }
-  }
+  RowSet<TX, VN, VPL, R> cur;
+  load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
   float g[VPL][VN], b[VPL][VN];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
     const int idx = lane + kWave * j;
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      g[j][k] = 0.f;
+      b[j][k] = 0.f;
+    }
     if (idx < nvec) {
       load_n<TP, VN>(gamma + idx * VN, g[j]);
-      if (beta) {
-        load_n<TP, VN>(beta + idx * VN, b[j]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < VN; ++k) b[j][k] = 0.f;
-      }
-    } else {
-#pragma unroll
-      for (int k = 0; k < VN; ++k) {
-        g[j][k] = 0.f;
-        b[j][k] = 0.f;
-      }
+      if (beta) load_n<TP, VN>(beta + idx * VN, b[j]);
     }
   }
   const float inv_c = 1.0f / (float)C;
+  for (; row0 < rows; row0 += step) {
+    RowSet<TX, VN, VPL, R> nxt;
+    if (row0 + step < rows) load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
+    // the R rows are independent: their reductions interleave
+    float mu[R], rs[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    if (row0 + r >= rows) break;
-    float s = 0.f;
+    for (int r = 0; r < R; ++r) {
+      float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < VPL; ++j)
+      for (int j = 0; j < VPL; ++j)
 #pragma unroll
-      for (int k = 0; k < VN; ++k) s += raw_get<TX, VN>(xr[r][j], k);
-    const float mu = wave_reduce(s, SumOp{}) * inv_c;
-    float q = 0.f;
+        for (int k = 0; k < VN; ++k) s += raw_get<TX, VN>(cur.v[r][j], k);
+      mu[r] = s;
+    }
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      if (lane + kWave * j < nvec) {
+    for (int r = 0; r < R; ++r) mu[r] = wave_reduce(mu[r], SumOp{}) * inv_c;
 #pragma unroll
-        for (int k = 0; k < VN; ++k) {
-          const float d = raw_get<TX, VN>(xr[r][j], k) - mu;
-          q += d * d;
+    for (int r = 0; r < R; ++r) {
+      float q = 0.f;
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        if (lane + kWave * j < nvec) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k) {
+            const float d = raw_get<TX, VN>(cur.v[r][j], k) - mu[r];
+            q += d * d;
+          }
+        }
+      }
+      rs[r] = q;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) rs[r] = 1.0f / sqrtf(wave_reduce(rs[r], SumOp{}) * inv_c + eps);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (row0 + r >= rows) break;
+      if (lane == 0) {
+        mean[row0 + r] = mu[r];
+        rstd[row0 + r] = rs[r];
+      }
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int idx = lane + kWave * j;
+        if (idx < nvec) {
+          float o[VN];
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            o[k] = (raw_get<TX, VN>(cur.v[r][j], k) - mu[r]) * rs[r] * g[j][k] + b[j][k];
+          store_n<TY, VN>(y + (row0 + r) * C + (int64_t)idx * VN, o);
         }
       }
     }
-    const float var = wave_reduce(q, SumOp{}) * inv_c;
-    const float rs = 1.0f / sqrtf(var + eps);
-    if (lane == 0) {
-      mean[row0 + r] = mu;
-      rstd[row0 + r] = rs;
-    }
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      const int idx = lane + kWave * j;
-      if (idx < nvec) {
-        float o[VN];
-#pragma unroll
-        for (int k = 0; k < VN; ++k)
-          o[k] = (raw_get<TX, VN>(xr[r][j], k) - mu) * rs * g[j][k] + b[j][k];
-        store_n<TY, VN>(y + (row0 + r) * C + (int64_t)idx * VN, o);
-      }
-    }
+    cur = nxt;
   }
 }
 
 // ----------------------------------------------------------- fast backward
+// Same walk as the forward kernel, with dy and x prefetched one step ahead.
 template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int R, bool HAS_DX,
           bool HAS_DP>
 __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
@@ -185,7 +213,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
   const int wave = threadIdx.x >> 6;
   constexpr int kWaves = kLnThreads / kWave;
   const int64_t gw = (int64_t)blockIdx.x * kWaves + wave;
-  const int64_t n_waves = (int64_t)gridDim.x * kWaves;
+  const int64_t step = (int64_t)gridDim.x * kWaves * R;
   const int nvec = C / VN;
   const float inv_c = 1.0f / (float)C;
 
@@ -201,27 +229,32 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
     if (HAS_DX && lane + kWave * j < nvec) load_n<TP, VN>(gamma + (lane + kWave * j) * VN, g[j]);
   }
 
-  for (int64_t row0 = gw * R; row0 < rows; row0 += n_waves * R) {
-    Raw<TDY, VN> dr[R][VPL];
-    Raw<TX, VN> xr[R][VPL];
-    float mu[R], rs[R];
+  int64_t row0 = gw * R;
+  RowSet<TDY, VN, VPL, R> dcur;
+  RowSet<TX, VN, VPL, R> xcur;
+  float mu[R], rs[R];
+  if (row0 < rows) {
+    load_rows<TDY, VN, VPL, R>(dcur, dy, row0, rows, C, nvec, lane);
+    load_rows<TX, VN, VPL, R>(xcur, x, row0, rows, C, nvec, lane);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const bool live = row0 + r < rows;
+      mu[r] = row0 + r < rows ? mean[row0 + r] : 0.f;
+      rs[r] = row0 + r < rows ? rstd[row0 + r] : 0.f;
+    }
+  }
+  for (; row0 < rows; row0 += step) {
+    RowSet<TDY, VN, VPL, R> dnxt;
+    RowSet<TX, VN, VPL, R> xnxt;
+    float nmu[R], nrs[R];
+    const int64_t nrow0 = row0 + step;
+    if (nrow0 < rows) {
+      load_rows<TDY, VN, VPL, R>(dnxt, dy, nrow0, rows, C, nvec, lane);
+      load_rows<TX, VN, VPL, R>(xnxt, x, nrow0, rows, C, nvec, lane);
 #pragma unroll
-      for (int j = 0; j < VPL; ++j) {
-        const int idx = lane + kWave * j;
-        if (live && idx < nvec) {
-          const int64_t off = (row0 + r) * C + (int64_t)idx * VN;
-          dr[r][j] = load_raw<TDY, VN>(dy + off);
-          xr[r][j] = load_raw<TX, VN>(x + off);
-        } else {
-          dr[r][j] = zero_raw<TDY, VN>();
-          xr[r][j] = zero_raw<TX, VN>();
-        }
+      for (int r = 0; r < R; ++r) {
+        nmu[r] = nrow0 + r < rows ? mean[nrow0 + r] : 0.f;
+        nrs[r] = nrow0 + r < rows ? rstd[nrow0 + r] : 0.f;
       }
-      mu[r] = live ? mean[row0 + r] : 0.f;
-      rs[r] = live ? rstd[row0 + r] : 0.f;
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -232,9 +265,9 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
       for (int j = 0; j < VPL; ++j) {
 #pragma unroll
         for (int k = 0; k < VN; ++k) {
-          // lanes past the row hold zeros in dr, so they add nothing
-          xh[j][k] = (raw_get<TX, VN>(xr[r][j], k) - mu[r]) * rs[r];
-          dv[j][k] = raw_get<TDY, VN>(dr[r][j], k);
+          // lanes past the row hold zeros in dy, so they add nothing
+          xh[j][k] = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
+          dv[j][k] = raw_get<TDY, VN>(dcur.v[r][j], k);
           if constexpr (HAS_DP) {
             acc_g[j][k] += dv[j][k] * xh[j][k];
             acc_b[j][k] += dv[j][k];
@@ -261,6 +294,13 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
           }
         }
       }
+    }
+    dcur = dnxt;
+    xcur = xnxt;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      mu[r] = nmu[r];
+      rs[r] = nrs[r];
     }
   }
 
@@ -289,9 +329,10 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
   }
 }
 
-// Adds `nparts` partial rows in ascending order.  grid (ceil(C/64), 2),
-// block (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one
-// column, then row 0 of the block adds the 16 sub-sums in order.
+// Adds `nparts` partial rows in a fixed order.  grid (ceil(C/64), 2), block
+// (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one column
+// into four interleaved accumulators (so four loads are always in flight),
+// then row 0 of the block adds the 16 sub-sums in order.
 template <typename TP>
 __global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__restrict__ partial,
                                                                int nparts, TP *__restrict__ dgamma,
@@ -304,7 +345,20 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__re
   const int col = blockIdx.x * 64 + threadIdx.x;
   float s = 0.f;
   if (col < C) {
-    for (int p = threadIdx.y; p < nparts; p += 16) s += partial[((int64_t)p * 2 + which) * C + col];
+    const float *src = partial + (int64_t)which * C + col;
+    const int64_t stride = 2 * (int64_t)C;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int p = threadIdx.y;
+    for (; p + 48 < nparts; p += 64) {
+      const float v0 = src[(int64_t)p * stride], v1 = src[(int64_t)(p + 16) * stride];
+      const float v2 = src[(int64_t)(p + 32) * stride], v3 = src[(int64_t)(p + 48) * stride];
+      a0 += v0;
+      a1 += v1;
+      a2 += v2;
+      a3 += v3;
+    }
+    for (; p < nparts; p += 16) a0 += src[(int64_t)p * stride];
+    s = (a0 + a1) + (a2 + a3);
   }
   sub[threadIdx.y][threadIdx.x] = s;
   __syncthreads();
@@ -414,8 +468,9 @@ __global__ __launch_bounds__(256) void ln_bwd_param_general_kernel(
 
 // ---------------------------------------------------------------- dispatch
 struct FastPlan {
-  int vpl = 0;  // 0: not eligible
-  int rows_per_wave = 1;
+  int vpl = 0;       // 0: not eligible
+  int fwd_rows = 1;  // rows a wave normalises per step, forward
+  int bwd_rows = 1;  // the same, backward (it holds twice the data per row)
 };
 
 // x vectors per lane needed for C columns of x_dtype; the fast kernels are
@@ -428,23 +483,30 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
   const int64_t per_lane = ceil_div(nvec, (int64_t)kWave);
   if (per_lane <= 2) {
     p.vpl = 2;
-    p.rows_per_wave = 4;
+    p.fwd_rows = 4;
+    p.bwd_rows = 2;
   } else if (per_lane <= 4) {
     p.vpl = 4;
-    p.rows_per_wave = 2;
+    p.fwd_rows = 2;
+    p.bwd_rows = 1;
   } else if (per_lane <= 8) {
     p.vpl = 8;
-    p.rows_per_wave = 1;
+    p.fwd_rows = 1;
+    p.bwd_rows = 1;
   }
   return p;
 }
 
-constexpr int kLnBwdMaxBlocks = 1024;
+// Grid caps: beyond these the waves loop over rows (with prefetch) instead of
+// the grid growing, which keeps the parameters in registers for many rows
+// and bounds the number of partial rows the backward pass leaves behind.
+constexpr int kLnFwdMaxBlocks = 1024;
+constexpr int kLnBwdMaxBlocks = 512;
 
-int ln_bwd_blocks(int64_t rows, const FastPlan &p) {
-  const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * p.rows_per_wave;
+int ln_blocks(int64_t rows, int rows_per_wave, int cap) {
+  const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * rows_per_wave;
   const int64_t b = ceil_div(rows, rows_per_block);
-  return (int)(b < kLnBwdMaxBlocks ? b : kLnBwdMaxBlocks);
+  return (int)(b < cap ? b : cap);
 }
 
 template <typename TX, typename TY, typename TP>
@@ -453,10 +515,7 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
-      const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * p.rows_per_wave;
-      const int64_t blocks = ceil_div(rows, rows_per_block);
-      if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
-      const dim3 grid((unsigned)blocks), block(kLnThreads);
+      const dim3 grid((unsigned)ln_blocks(rows, p.fwd_rows, kLnFwdMaxBlocks)), block(kLnThreads);
 #define CS_LN_FWD(VPL, R)                                                                   \
   ln_fwd_rows_kernel<TX, TY, TP, VPL, R><<<grid, block, 0, s>>>(                            \
       (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean,           \
@@ -489,7 +548,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
-      const int blocks = ln_bwd_blocks(rows, p);
+      const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks);
       const size_t need = want_dp ? (size_t)blocks * 2 * C * sizeof(float) : 0;
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
       const size_t lds = want_dp ? (size_t)(kLnThreads / kWave) * C * sizeof(float) : 0;
@@ -507,9 +566,9 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
     CS_LN_BWD(VPL, R, false, true);           \
   }
       if (p.vpl == 2) {
-        CS_LN_BWD_MASK(2, 4)
+        CS_LN_BWD_MASK(2, 2)
       } else if (p.vpl == 4) {
-        CS_LN_BWD_MASK(4, 2)
+        CS_LN_BWD_MASK(4, 1)
       } else {
         CS_LN_BWD_MASK(8, 1)
       }
@@ -589,12 +648,8 @@ extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void
 
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
-  // the fast path's largest grid: the narrowest plan has the fewest rows per
-  // block, so it bounds every dtype
-  FastPlan p;
-  p.vpl = 8;
-  p.rows_per_wave = 1;
-  return (size_t)ln_bwd_blocks(rows, p) * 2 * (size_t)C * sizeof(float);
+  // the fast path's largest grid: one row per wave per step
+  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks) * 2 * (size_t)C * sizeof(float);
 }
 
 extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *mean,

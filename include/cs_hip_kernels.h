@@ -73,6 +73,13 @@ enum cs_error {
 int cs_hip_abi_version(void);
 const char *cs_hip_error_string(int code);
 
+/* Plain device-to-device copy of `bytes` (a multiple of 16, both pointers
+ * 16-byte aligned) with the same 16-byte streaming accesses the ops use.  It
+ * has no counterpart in the reference: it is the calibration kernel of the
+ * benchmark (the bandwidth a trivial HBM-bound kernel reaches on this device,
+ * and the scale of the hardware traffic counters). */
+int cs_stream_copy(void *dst, const void *src, int64_t bytes, void *stream);
+
 /* ------------------------------------------------------------------------
  * AdamW
  * replaces stepKernel / stepKernelAmsgrad and the step<UpT,T> kernels,
