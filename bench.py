@@ -73,6 +73,12 @@ def hold_gpu(torch, ms=3.0):
         _capi.load().cs_stream_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), 1 << 30, st)
 
 
+def _capi_lib():
+    from core_scheduler_amd import _capi
+
+    return _capi.load()
+
+
 def event_ms(fn, reps, torch):
     """Median / mean duration of one call, each bracketed by its own pair of events."""
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
@@ -158,6 +164,11 @@ def per_op_table(args, torch, ops):
         return (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean).to(dtype)
 
     only = [o for o in args.ops.split(",") if o]
+    lib = _capi_lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def stream_copy(dst, src):
+        lib.cs_stream_copy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), src.numel(), stream)
 
     def wanted(name):
         return not only or any(name.startswith(o) for o in only)
@@ -185,6 +196,18 @@ def per_op_table(args, torch, ops):
             f"{rec['gbps_cold']:8.1f} GB/s  {rec['frac_cold']*100:5.1f}% of HBM peak")
         del sets
         torch.cuda.empty_cache()
+
+    # ---- calibration: a plain copy moving the same number of bytes as the ops below (half read,
+    # half written).  What it reaches is the practical ceiling at that size.
+    for mb in (25, 100, 400, 1600, 3500):
+        nbytes = int(mb * 1e6) // 32 * 32
+
+        def mk(nb=nbytes):
+            return {"a": torch.empty(nb // 2, dtype=torch.uint8, device=dev),
+                    "b": torch.empty(nb // 2, dtype=torch.uint8, device=dev)}
+
+        add("stream_copy", f"{mb} MB moved", nbytes, mk,
+            lambda s_: stream_copy(s_["b"], s_["a"]))
 
     # ---- configuration 3: LayerNorm [8192,768] bf16, fp32 parameters
     for tag, rows, C in (("small", 8192, 768), ("xl", 16384, 1600)):
@@ -334,6 +357,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-xl-adamw", dest="xl_adamw", action="store_false", help="skip the 25 GB XL AdamW line")
     ap.add_argument("--no-xl-ce", dest="xl_ce", action="store_false")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="K",
+                    help="also run K plain 1 GiB copies (to scale hardware traffic counters)")
     ap.add_argument("--cpu-rows", type=int, default=CE_N)
     ap.add_argument("--cpu-reps", type=int, default=5)
     args = ap.parse_args()
@@ -357,6 +382,17 @@ def main():
     value = CE_BYTES * args.steps / head["seconds"] / 1e9
     log(f"[bench] fused classifier: {head['ms_per_step']:.4f} ms/step wall, row kernel {head['rows_kernel_ms_avg']:.4f} ms "
         f"(events), {achieved:.0f} GB/s = {achieved / HBM_PEAK_GBPS * 100:.1f}% of HBM peak, loss {head['loss']:.4f}")
+
+    if args.calibrate_copy:
+        # a known-size kernel next to the row pass, for scaling hardware traffic counters
+        a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+        b = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(args.calibrate_copy):
+            capi.check("cs_stream_copy", capi.load().cs_stream_copy(ctypes.c_void_p(b.data_ptr()),
+                                                                      ctypes.c_void_p(a.data_ptr()), 1 << 30, st))
+        torch.cuda.synchronize()
+        del a, b
 
     table = [] if args.no_per_op else per_op_table(args, torch, ops)
     cpu = None
