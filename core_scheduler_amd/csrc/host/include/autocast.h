@@ -1,0 +1,19 @@
+// RAII switch for ATen autocast on the submitting thread (the reference's include/autocast.h).
+// The ops below consult at::autocast::is_enabled() the way ATen's own policy would apply to
+// the calls the reference makes: LayerNorm and the cross-entropy gradient come out in fp32.
+#pragma once
+#include <ATen/core/TensorBody.h>
+
+#include "export.h"
+#include "threading/scheduler.h"
+
+namespace cs::autocast {
+struct CS_API ContextGuard {
+  ContextGuard(const Scheduler &scheduler, at::ScalarType dtype);
+  ~ContextGuard();
+
+ private:
+  bool previous_;
+  at::ScalarType previous_dtype_;
+};
+}  // namespace cs::autocast

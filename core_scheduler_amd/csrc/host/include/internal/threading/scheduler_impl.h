@@ -1,0 +1,16 @@
+// Scheduler implementation interface (the reference's include/internal/threading/scheduler_impl.h).
+#pragma once
+#include "threading/scheduler.h"
+#include "threading/task.h"
+
+namespace cs {
+struct Scheduler::Impl {
+  explicit Impl(int64_t deviceRank) : device_rank_{deviceRank} {}
+  virtual ~Impl() = default;
+  virtual void submit(Task &&task);
+  [[nodiscard]] int64_t device_rank() const { return device_rank_; }
+
+ protected:
+  const int64_t device_rank_;
+};
+}  // namespace cs

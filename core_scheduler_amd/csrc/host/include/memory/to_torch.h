@@ -1,0 +1,13 @@
+// Copy of a cs tensor as an at::Tensor (the reference's test helper, include/memory/to_torch.h).
+#pragma once
+#include <ATen/core/TensorBody.h>
+
+#include "tensor.h"
+#include "threading/scheduler.h"
+
+namespace cs::memory {
+CS_API at::Tensor to_torch(const Scheduler &scheduler, const ReadOnlyTensor &tensor);
+// The other direction, for callers that already hold device data: a task that makes `handle`
+// refer to `tensor` (no copy).
+CS_API Tensor from_torch(const Scheduler &scheduler, const at::Tensor &tensor);
+}  // namespace cs::memory

@@ -1,0 +1,59 @@
+// cs::optimizer::AdamW, the reference's optimizer interface (include/optimizer/adamw.h:33-75).
+#pragma once
+#include <vector>
+
+#include "arg.h"
+#include "module/state.h"
+#include "tensor.h"
+#include "threading/scheduler.h"
+
+namespace cs::optimizer {
+struct CS_API AdamW {
+  AdamW() = delete;
+
+  struct State final : module::OptimizerState {
+    struct Tensors {
+      Tensor m;
+      Tensor v;
+      Tensor v_max{};
+    } tensors;
+    struct Options {
+      mutable double lr = 1e-3;
+      const double beta1 = 0.9;
+      const double beta2 = 0.999;
+      const double eps = 1e-8;
+      const double weight_decay = 1e-2;
+      const bool amsgrad = false;
+      long t = 0;
+    } options;
+
+    State(const Tensors &tensors, const Options &options);
+    void set_lr(double lr) const override;
+    double get_lr() const override;
+  };
+
+  struct Options {
+    CS_ARG(double, lr) = 1e-3;
+    CS_ARG(double, beta1) = 0.9;
+    CS_ARG(double, beta2) = 0.999;
+    CS_ARG(double, eps) = 1e-8;
+    CS_ARG(double, weight_decay) = 1e-2;
+    CS_ARG(bool, amsgrad) = false;
+    CS_ARG(long, t) = 0;
+  };
+
+  static std::shared_ptr<State> init(const Scheduler &scheduler, const ReadOnlyTensor &parameter,
+                                     const Options &options);
+
+  static void step(const Scheduler &scheduler, const std::shared_ptr<module::OptimizerState> &state,
+                   const Tensor &w, const ReadOnlyTensor &dw);
+
+  // Not in the reference: every parameter of a model in one task and one kernel launch
+  // (the loop of src/module/adamw.cpp:32-38).  All states must share hyper-parameters and
+  // step count; parameters with an undefined gradient are skipped with a warning, as the
+  // single-tensor step does.
+  static void step(const Scheduler &scheduler,
+                   const std::vector<std::shared_ptr<module::OptimizerState>> &states,
+                   const std::vector<Tensor> &ws, const std::vector<ReadOnlyTensor> &dws);
+};
+}  // namespace cs::optimizer

@@ -1,0 +1,177 @@
+// Python binding of the host API, so that the parity tests can drive cs::compute /
+// cs::optimizer exactly as the reference's gtest suites do: build a DynamicScheduler, init an
+// op state, call forward / backward, wait on the returned handles and compare.
+#include <torch/extension.h>
+
+#include <memory>
+#include <optional>
+#include <string>
+#include <vector>
+
+#include "autocast.h"
+#include "compute/cross_entropy.h"
+#include "compute/embedding.h"
+#include "compute/gelu.h"
+#include "compute/layer_norm.h"
+#include "memory/to_torch.h"
+#include "optimizer/adamw.h"
+#include "tensor_impl.h"
+#include "threading/dynamic_scheduler.h"
+
+namespace py = pybind11;
+using namespace cs;
+
+namespace {
+at::ScalarType dtype_from(const std::string &name) {
+  if (name == "float32") return at::kFloat;
+  if (name == "float64") return at::kDouble;
+  if (name == "float16") return at::kHalf;
+  if (name == "bfloat16") return at::kBFloat16;
+  throw std::invalid_argument("unknown dtype " + name);
+}
+Tensor as_tensor(const ReadOnlyTensor &t) {
+  Tensor out;
+  static_cast<ReadOnlyTensor &>(out) = t;
+  return out;
+}
+c10::DeviceIndex device_of(const Scheduler &s) {
+  return static_cast<c10::DeviceIndex>(s.impl() ? s.get_device_rank() : 0);
+}
+struct AutocastScope {
+  std::unique_ptr<autocast::ContextGuard> guard;
+};
+}  // namespace
+
+PYBIND11_MODULE(_cs_host, m) {
+  m.doc() = "cs::compute / cs::optimizer host API over the gfx950 kernel library";
+
+  // a bare Scheduler has no implementation behind it; it exists so that argument checks that
+  // fail before any task is submitted can be exercised without a device
+  py::class_<Scheduler>(m, "Scheduler").def(py::init<>()).def("get_device_rank", &Scheduler::get_device_rank);
+  py::class_<DynamicScheduler, Scheduler>(m, "DynamicScheduler").def(py::init<int>(), py::arg("local_rank"));
+
+  py::class_<ReadOnlyTensor>(m, "ReadOnlyTensor")
+      .def("wait", &ReadOnlyTensor::wait)
+      .def("numel", &ReadOnlyTensor::numel)
+      .def("defined", [](const ReadOnlyTensor &t) { return t.impl()->tensor().defined(); })
+      .def("sizes", [](const ReadOnlyTensor &t) { return t.sizes().vec(); })
+      .def("priority", [](const ReadOnlyTensor &t) { return static_cast<int>(t.impl()->priority()); });
+  py::class_<Tensor, ReadOnlyTensor>(m, "Tensor").def(py::init<>());
+
+  m.def("to_torch", &memory::to_torch, py::arg("scheduler"), py::arg("tensor"));
+  m.def("from_torch", &memory::from_torch, py::arg("scheduler"), py::arg("tensor"));
+
+  py::class_<AutocastScope>(m, "autocast")
+      .def(py::init([]() { return AutocastScope{}; }))
+      .def("enter",
+           [](AutocastScope &s, const Scheduler &sched, const std::string &dtype) {
+             s.guard = std::make_unique<autocast::ContextGuard>(sched, dtype_from(dtype));
+           })
+      .def("exit", [](AutocastScope &s) { s.guard.reset(); });
+
+  // ---- GeLU
+  {
+    using Op = compute::GeLU;
+    py::class_<Op::State, std::shared_ptr<Op::State>>(m, "GeLUState");
+    auto sub = m.def_submodule("GeLU");
+    sub.def("init", [](const Scheduler &s, int approximate) {
+      return approximate == 0 ? Op::init(s) : Op::init(s, Op::Options{}.approximate(approximate));
+    }, py::arg("scheduler"), py::arg("approximate") = 0);
+    sub.def("forward", &Op::forward);
+    sub.def("backward", &Op::backward);
+  }
+  // ---- CrossEntropy
+  {
+    using Op = compute::CrossEntropy;
+    py::class_<Op::State, std::shared_ptr<Op::State>>(m, "CrossEntropyState")
+        .def("total_weight", [](const Op::State &s) { return as_tensor(s.backward.total_weight); });
+    auto sub = m.def_submodule("CrossEntropy");
+    sub.def("init", [](const Scheduler &s, int reduction, int64_t ignore_index, double label_smoothing,
+                       int64_t num_classes) {
+      return Op::init(s, Op::Options{}
+                             .reduction(static_cast<at::Reduction::Reduction>(reduction))
+                             .ignore_index(ignore_index)
+                             .label_smoothing(label_smoothing)
+                             .num_classes(num_classes));
+    }, py::arg("scheduler"), py::arg("reduction") = 1, py::arg("ignore_index") = -100,
+            py::arg("label_smoothing") = 0.0, py::arg("num_classes") = -1);
+    sub.def("forward", &Op::forward);
+    sub.def("backward", &Op::backward);
+  }
+  // ---- LayerNorm
+  {
+    using Op = compute::LayerNorm;
+    py::class_<Op::State, std::shared_ptr<Op::State>>(m, "LayerNormState")
+        .def_property_readonly("weight", [](const Op::State &s) { return s.forward.weight; })
+        .def_property_readonly("bias", [](const Op::State &s) { return s.forward.bias; })
+        .def_property_readonly("grad_weight", [](const Op::State &s) { return s.forward.grad_weight; })
+        .def_property_readonly("grad_bias", [](const Op::State &s) { return s.forward.grad_bias; })
+        .def("set_weight", [](Op::State &s, const Tensor &t) { s.forward.weight = t; })
+        .def("set_bias", [](Op::State &s, const Tensor &t) { s.forward.bias = t; })
+        .def("parameter_names", [](const Op::State &s) { return s.parameters().keys(); })
+        .def("zero_grad", &Op::State::zero_grad);
+    auto sub = m.def_submodule("LayerNorm");
+    sub.def("init", [](const Scheduler &s, std::vector<int64_t> shape, double eps, bool affine, bool bias,
+                       const std::string &dtype) {
+      return Op::init(s, Op::Options{shape}.eps(eps).elementwise_affine(affine).bias(bias)
+                             .device(at::Device(at::kCUDA, device_of(s)))
+                             .dtype(dtype_from(dtype)));
+    }, py::arg("scheduler"), py::arg("normalized_shape"), py::arg("eps") = 1e-5,
+            py::arg("elementwise_affine") = true, py::arg("bias") = true, py::arg("dtype") = "float32");
+    sub.def("forward", &Op::forward);
+    sub.def("backward", &Op::backward);
+  }
+  // ---- Embedding
+  {
+    using Op = compute::Embedding;
+    py::class_<Op::State, std::shared_ptr<Op::State>>(m, "EmbeddingState")
+        .def_property_readonly("weight", [](const Op::State &s) { return s.forward.weight; })
+        .def_property_readonly("grad_weight", [](const Op::State &s) { return s.forward.grad_weight; })
+        .def_property_readonly("padding_idx", [](const Op::State &s) { return s.args.padding_idx; })
+        .def("set_weight", [](Op::State &s, const Tensor &t) { s.forward.weight = t; })
+        .def("zero_grad", &Op::State::zero_grad);
+    auto sub = m.def_submodule("Embedding");
+    sub.def("init", [](const Scheduler &s, int64_t n, int64_t d, std::optional<int64_t> padding_idx,
+                       std::optional<double> max_norm, const std::string &dtype) {
+      auto o = Op::Options{n, d}
+                   .device(at::Device(at::kCUDA, device_of(s)))
+                   .dtype(dtype_from(dtype));
+      if (padding_idx) o = o.padding_idx(*padding_idx);
+      if (max_norm) o = o.max_norm(*max_norm);
+      return Op::init(s, o);
+    }, py::arg("scheduler"), py::arg("num_embeddings"), py::arg("embedding_dim"),
+            py::arg("padding_idx") = py::none(), py::arg("max_norm") = py::none(), py::arg("dtype") = "float32");
+    sub.def("forward", &Op::forward);
+    sub.def("backward", &Op::backward);
+    sub.def("forward_with_positions", &Op::forward_with_positions);
+    sub.def("backward_with_positions", &Op::backward_with_positions);
+  }
+  // ---- AdamW
+  {
+    using Op = optimizer::AdamW;
+    py::class_<module::OptimizerState, std::shared_ptr<module::OptimizerState>>(m, "OptimizerState")
+        .def("set_lr", &module::OptimizerState::set_lr)
+        .def("get_lr", &module::OptimizerState::get_lr);
+    py::class_<Op::State, module::OptimizerState, std::shared_ptr<Op::State>>(m, "AdamWState")
+        .def_property_readonly("m", [](const Op::State &s) { return s.tensors.m; })
+        .def_property_readonly("v", [](const Op::State &s) { return s.tensors.v; })
+        .def_property_readonly("v_max", [](const Op::State &s) { return s.tensors.v_max; })
+        .def_property_readonly("t", [](const Op::State &s) { return s.options.t; });
+    auto sub = m.def_submodule("AdamW");
+    sub.def("init", [](const Scheduler &s, const ReadOnlyTensor &p, double lr, double beta1, double beta2, double eps,
+                       double weight_decay, bool amsgrad, long t) {
+      return Op::init(s, p, Op::Options{}.lr(lr).beta1(beta1).beta2(beta2).eps(eps).weight_decay(weight_decay)
+                                .amsgrad(amsgrad).t(t));
+    }, py::arg("scheduler"), py::arg("parameter"), py::arg("lr") = 1e-3, py::arg("beta1") = 0.9,
+            py::arg("beta2") = 0.999, py::arg("eps") = 1e-8, py::arg("weight_decay") = 1e-2,
+            py::arg("amsgrad") = false, py::arg("t") = 0);
+    sub.def("step", [](const Scheduler &s, const std::shared_ptr<Op::State> &state, const Tensor &w,
+                       const ReadOnlyTensor &dw) { Op::step(s, state, w, dw); });
+    sub.def("step_all", [](const Scheduler &s, const std::vector<std::shared_ptr<Op::State>> &states,
+                           const std::vector<Tensor> &ws, const std::vector<Tensor> &dws) {
+      std::vector<std::shared_ptr<module::OptimizerState>> base(states.begin(), states.end());
+      std::vector<ReadOnlyTensor> grads(dws.begin(), dws.end());
+      Op::step(s, base, ws, grads);
+    });
+  }
+}

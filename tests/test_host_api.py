@@ -1,0 +1,298 @@
+"""The C++ host API (cs::compute / cs::optimizer over the C ABI), driven the way the reference's
+gtest suites drive theirs: a DynamicScheduler, op states, forward / backward, wait, compare.
+
+Cases follow test/test_gelu.cpp, test_embedding.cpp, test_cross_entropy.cpp, test_layer_norm.cpp,
+test_adamw.cpp and test_autocast.cpp of the reference; expected values come from the CPU oracle.
+The error-convention tests at the bottom need no GPU.
+"""
+import os
+import subprocess
+import sys
+import textwrap
+
+import pytest
+import torch
+
+from _util import assert_bit_exact, assert_close, randint, randn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def host():
+    from core_scheduler_amd import _cs_host
+
+    return _cs_host
+
+
+@pytest.fixture(scope="module")
+def sched(host):
+    return host.DynamicScheduler(0)
+
+
+@pytest.fixture(scope="module")
+def co():
+    from oracle import c_oracle
+
+    return c_oracle
+
+
+def up(host, sched, t):
+    return host.from_torch(sched, t.to(DEV))
+
+
+def down(host, sched, handle):
+    return host.to_torch(sched, handle).cpu()
+
+
+# ---------------------------------------------------------------------------- GeLU
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("T", [128, 512, 1024])
+def test_gelu_routine(host, sched, co, dtype, T):
+    # test/test_gelu.cpp:59-102: B 2, d 512 (smaller here), randn input, randn grad_output
+    x = randn((2, T, 256), 1, dtype=dtype)
+    dy = randn((2, T, 256), 2, dtype=dtype)
+    state = host.GeLU.init(sched)
+    y = host.GeLU.forward(sched, state, up(host, sched, x))
+    dx = host.GeLU.backward(sched, state, up(host, sched, dy))
+    y.wait()
+    assert_close(down(host, sched, y), co.gelu_forward(x), atol=1e-6, name="y")
+    assert_close(down(host, sched, dx), co.gelu_backward(dy, x), atol=5e-6, name="dx")
+    # the tanh form is an option the reference does not have
+    state = host.GeLU.init(sched, approximate=1)
+    y = host.GeLU.forward(sched, state, up(host, sched, x))
+    assert_close(down(host, sched, y), co.gelu_forward(x, "tanh"), atol=1e-6, name="y tanh")
+
+
+# ----------------------------------------------------------------------- Embedding
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_embedding_routine(host, sched, co, dtype):
+    # test/test_embedding.cpp:58-97: B 2, T 1024, vocab 4095, d 512, int32 ids in [0, 3)
+    B, T, V, d = 2, 1024, 4095, 512
+    tdt = getattr(torch, dtype)
+    ids = randint(0, 3, (B, T), 3, dtype=torch.int32)
+    state = host.Embedding.init(sched, V, d, dtype=dtype)
+    w = down(host, sched, state.weight)
+    assert w.shape == (V, d) and w.dtype == tdt and abs(w.float().std().item() - 1) < 0.05  # N(0, 1) init
+    out = host.Embedding.forward(sched, state, up(host, sched, ids))
+    out.wait()
+    got = down(host, sched, out)
+    assert got.shape == (B, T, d)
+    assert_bit_exact(got, co.embedding_forward(w, ids), "forward")
+    dout = randn((B, T, d), 4, dtype=tdt)
+    assert not state.grad_weight.defined()
+    host.Embedding.backward(sched, state, up(host, sched, dout))
+    want = co.embedding_backward(dout, ids, V)
+    assert state.grad_weight.priority() == 1  # produced on the assist stream, as in the reference
+    assert_close(down(host, sched, state.grad_weight), want, atol=2e-5 if dtype == "float32" else 1e-6, name="grad")
+    # a second backward accumulates (`+=`), zero_grad drops the gradient
+    host.Embedding.forward(sched, state, up(host, sched, ids))
+    host.Embedding.backward(sched, state, up(host, sched, dout))
+    assert_close(down(host, sched, state.grad_weight), co.embedding_backward(dout, ids, V, dweight=want),
+                 atol=4e-5 if dtype == "float32" else 1e-6, name="grad +=")
+    state.zero_grad()
+    assert not state.grad_weight.defined()
+
+
+@pytest.mark.gpu
+def test_embedding_with_positions(host, sched, co):
+    B, T, V, C = 4, 64, 500, 128
+    tok = host.Embedding.init(sched, V, C, dtype="bfloat16")
+    pos = host.Embedding.init(sched, T, C, dtype="bfloat16")
+    wte, wpe = down(host, sched, tok.weight), down(host, sched, pos.weight)
+    ids = randint(0, V, (B, T), 5)
+    out = host.Embedding.forward_with_positions(sched, tok, pos, up(host, sched, ids))
+    assert_bit_exact(down(host, sched, out), co.embedding_forward_add(wte, wpe, ids), "gather-add")
+    dout = randn((B, T, C), 6, dtype=torch.bfloat16)
+    host.Embedding.backward_with_positions(sched, tok, pos, up(host, sched, dout))
+    assert_close(down(host, sched, tok.grad_weight), co.embedding_backward(dout, ids, V), atol=1e-6, name="dwte")
+    assert_close(down(host, sched, pos.grad_weight), co.embedding_backward_positions(dout), atol=1e-6, name="dwpe")
+
+
+# ------------------------------------------------------------------- CrossEntropy
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_cross_entropy_routine(host, sched, co, dtype):
+    # test/test_cross_entropy.cpp:69-99: x = rand [B*256, 384] (B smaller here), int64 targets
+    N, V = 8 * 256, 384
+    x = torch.rand((N, V), generator=torch.Generator().manual_seed(1)).to(dtype)
+    t = randint(0, V, (N,), 7)
+    state = host.CrossEntropy.init(sched)
+    loss = host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t))
+    dx = host.CrossEntropy.backward(sched, state)
+    loss.wait()
+    want_loss, _, want_dx, _ = co.cross_entropy(x, t)
+    assert_close(down(host, sched, loss).double(), want_loss.double(), atol=1e-5, name="loss")
+    assert_close(down(host, sched, dx), want_dx, atol=1e-9, name="dx")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_cross_entropy_amp(host, sched, co, dtype):
+    # test/test_cross_entropy.cpp:102-139: 16-bit logits inside the autocast guard, fp32 gradient
+    N, V = 1024, 384
+    x = torch.rand((N, V), generator=torch.Generator().manual_seed(1)).to(getattr(torch, dtype))
+    t = randint(0, V, (N,), 8)
+    scope = host.autocast()
+    scope.enter(sched, dtype)
+    try:
+        state = host.CrossEntropy.init(sched)
+        loss = host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t))
+        dx = host.CrossEntropy.backward(sched, state)
+    finally:
+        scope.exit()
+    got = down(host, sched, dx)
+    assert got.dtype == torch.float32
+    want_loss, _, want_dx, _ = co.cross_entropy(x, t, dlogits_dtype=torch.float32)
+    assert_close(down(host, sched, loss), want_loss, atol=1e-5, name="loss")
+    assert_close(got, want_dx, atol=1e-9, name="dx fp32")
+    # outside the guard the gradient keeps the logits' dtype; padded vocabulary via num_classes
+    state = host.CrossEntropy.init(sched, num_classes=300)
+    host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t % 300))
+    got = down(host, sched, host.CrossEntropy.backward(sched, state))
+    assert got.dtype == x.dtype and (got[:, 300:] == 0).all()
+
+
+# ---------------------------------------------------------------------- LayerNorm
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_layer_norm_routine(host, sched, co, dtype):
+    # test/test_layer_norm.cpp:63-134: x = rand [.., 384], weight 1, bias 0
+    tdt = getattr(torch, dtype)
+    x = torch.rand((16, 64, 384), generator=torch.Generator().manual_seed(1)).to(tdt)
+    dy = torch.rand((16, 64, 384), generator=torch.Generator().manual_seed(2)).to(tdt)
+    state = host.LayerNorm.init(sched, [384], dtype=dtype)
+    assert list(state.parameter_names()) == ["weight", "bias"]
+    w, b = down(host, sched, state.weight), down(host, sched, state.bias)
+    assert (w == 1).all() and (b == 0).all()
+    y = host.LayerNorm.forward(sched, state, up(host, sched, x))
+    dx = host.LayerNorm.backward(sched, state, up(host, sched, dy))
+    y2, mean, rstd = co.layernorm_forward(x.reshape(-1, 384), w, b)
+    dx2, dg2, db2 = co.layernorm_backward(dy.reshape(-1, 384), x.reshape(-1, 384), mean, rstd, w)
+    tight = dtype == "float64"
+    assert_close(down(host, sched, y).reshape(-1, 384), y2, atol=1e-13 if tight else 2e-6, name="y")
+    assert_close(down(host, sched, dx).reshape(-1, 384), dx2, atol=1e-13 if tight else 5e-6, name="dx")
+    # column sums of 1024 terms of size ~0.5: fp32 rounding of the running sum allows about
+    # 2 * 6e-8 * (sum of the terms' magnitudes) = 1e-4 in absolute terms
+    assert_close(down(host, sched, state.grad_weight), dg2, atol=1e-10 if tight else 1e-4, name="dgamma")
+    assert_close(down(host, sched, state.grad_bias), db2, atol=1e-10 if tight else 1e-4, name="dbeta")
+    # second backward accumulates into the existing gradients (src/compute/layer_norm.cpp:325-334)
+    host.LayerNorm.forward(sched, state, up(host, sched, x))
+    host.LayerNorm.backward(sched, state, up(host, sched, dy))
+    assert_close(down(host, sched, state.grad_bias), 2 * db2, atol=1e-9 if tight else 2e-4, name="dbeta +=")
+    state.zero_grad()
+    assert not state.grad_weight.defined() and not state.grad_bias.defined()
+
+
+@pytest.mark.gpu
+def test_layer_norm_autocast_and_no_bias(host, sched, co):
+    # test/test_autocast.cpp:112-156: bf16 x inside the guard, fp32 parameters, fp32 y and dy
+    x = randn((8, 64, 768), 9, dtype=torch.bfloat16)
+    dy = randn((8, 64, 768), 10)
+    state = host.LayerNorm.init(sched, [768], dtype="float32")
+    gamma, beta = randn(768, 11, std=0.02, mean=1.0), randn(768, 12, std=0.02)
+    state.set_weight(up(host, sched, gamma))
+    state.set_bias(up(host, sched, beta))
+    scope = host.autocast()
+    scope.enter(sched, "bfloat16")
+    try:
+        y = host.LayerNorm.forward(sched, state, up(host, sched, x))
+        dx = host.LayerNorm.backward(sched, state, up(host, sched, dy))
+    finally:
+        scope.exit()
+    got_y = down(host, sched, y)
+    assert got_y.dtype == torch.float32
+    y2, mean, rstd = co.layernorm_forward(x.reshape(-1, 768), gamma, beta, out_dtype=torch.float32)
+    dx2, dg2, db2 = co.layernorm_backward(dy.reshape(-1, 768), x.reshape(-1, 768), mean, rstd, gamma,
+                                          out_dtype=torch.float32)
+    assert_close(got_y.reshape(-1, 768), y2, atol=2e-6, name="y fp32")
+    assert_close(down(host, sched, dx).reshape(-1, 768), dx2, atol=5e-6, name="dx fp32")
+    assert_close(down(host, sched, state.grad_weight), dg2, atol=1e-4, name="dgamma")  # 512 terms of size ~1
+    assert_close(down(host, sched, state.grad_bias), db2, atol=1e-4, name="dbeta")
+    # bias=false path (src/compute/layer_norm.cpp:198-204)
+    nb = host.LayerNorm.init(sched, [768], bias=False, dtype="float32")
+    assert list(nb.parameter_names()) == ["weight"]
+    xs = randn((32, 768), 13)
+    y = host.LayerNorm.forward(sched, nb, up(host, sched, xs))
+    assert_close(down(host, sched, y), co.layernorm_forward(xs, torch.ones(768), None)[0], atol=2e-6, name="no bias")
+    host.LayerNorm.backward(sched, nb, up(host, sched, xs))
+    assert nb.grad_weight.defined() and not nb.grad_bias.defined()
+
+
+# -------------------------------------------------------------------------- AdamW
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", [128, 512, 1024])
+def test_adamw_functional_routine(host, sched, size):
+    # test/test_adamw.cpp:63-103, with the closed form and the tolerances written there
+    lr, b1, b2, eps, wd = 1.0, 0.9, 0.999, 1e-8, 1e-2
+    x0 = torch.rand(size, generator=torch.Generator().manual_seed(1))
+    dx = torch.rand(size, generator=torch.Generator().manual_seed(2))
+    x = up(host, sched, x0)
+    state = host.AdamW.init(sched, x, lr=lr, beta1=b1, beta2=b2, eps=eps, weight_decay=wd, t=0)
+    host.AdamW.step(sched, state, x, up(host, sched, dx))
+    assert state.t == 1
+    xt = x0 - lr * wd * x0
+    mt = (1 - b1) * dx
+    vt = (1 - b2) * dx.square()
+    xt = xt - lr * (mt / (1 - b1)) / ((vt / (1 - b2)).sqrt() + eps)
+    assert torch.allclose(down(host, sched, x), xt, 1e-4, 1e-5)
+    assert torch.allclose(down(host, sched, state.m), mt, 1e-4, 1e-5)
+    assert torch.allclose(down(host, sched, state.v), vt, 1e-4, 1e-5)
+
+
+@pytest.mark.gpu
+def test_adamw_all_parameters_in_one_task(host, sched, co):
+    # the loop of src/module/adamw.cpp:32-38 as one launch; compared with per-tensor steps and the oracle
+    hp = dict(lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    shapes = [(300, 64), (64,), (5000,), (17, 3)]
+    ws0 = [randn(s, 20 + i, std=0.02) for i, s in enumerate(shapes)]
+    gs = [randn(s, 40 + i, std=1e-3) for i, s in enumerate(shapes)]
+    ws = [up(host, sched, w) for w in ws0]
+    states = [host.AdamW.init(sched, w, **hp) for w in ws]
+    for _ in range(3):
+        host.AdamW.step_all(sched, states, ws, [up(host, sched, g) for g in gs])
+    states[0].set_lr(1e-3)
+    assert states[0].get_lr() == 1e-3
+    for i, s in enumerate(shapes):
+        w, m, v = ws0[i], torch.zeros(s), torch.zeros(s)
+        for t in range(1, 4):
+            w, m, v, _ = co.adamw_step(w, gs[i], m, v, t=t, **hp)
+        assert_close(down(host, sched, ws[i]), w.reshape(s), atol=1e-8, name=f"w[{i}]")
+        assert_close(down(host, sched, states[i].v), v.reshape(s), atol=1e-13, name=f"v[{i}]")
+    # an undefined gradient is skipped with a warning and leaves the parameter alone
+    before = down(host, sched, ws[1])
+    host.AdamW.step(sched, states[1], ws[1], host.Tensor())
+    assert_bit_exact(down(host, sched, ws[1]), before, "skipped update")
+
+
+# ------------------------------------------------------ error conventions (no GPU)
+def run_snippet(code):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    return subprocess.run([sys.executable, "-c", textwrap.dedent(code)], capture_output=True, text=True, env=env,
+                          timeout=120)
+
+
+def test_label_smoothing_aborts_like_the_reference():
+    # src/compute/cross_entropy.cpp:30-31: CS_ASSERT_TRUE -> log critical + std::abort
+    p = run_snippet("""
+        from core_scheduler_amd import _cs_host as h
+        h.CrossEntropy.init(h.Scheduler(), 1, -100, 0.1, -1)
+    """)
+    assert p.returncode != 0 and "label_smoothing" in (p.stderr + p.stdout)
+
+
+def test_embedding_argument_checks_raise():
+    # src/compute/embedding.cpp:80-92: TORCH_CHECK on padding_idx and max_norm
+    p = run_snippet("""
+        from core_scheduler_amd import _cs_host as h
+        s = h.Scheduler()
+        for kwargs in (dict(padding_idx=10), dict(padding_idx=-11), dict(max_norm=1.0)):
+            try:
+                h.Embedding.init(s, 10, 4, **kwargs)
+            except RuntimeError as e:
+                print("raised:", str(e).splitlines()[0])
+    """)
+    assert p.stdout.count("raised:") == 3, p.stdout + p.stderr
