@@ -10,7 +10,8 @@
 // cycles per element forward, which libm's tanhf would exceed, so 16-bit
 // storage uses the identity 0.5*(1+tanh(u)) = 1/(1+exp(-2u)) with the hardware
 // exp2 and reciprocal (1 ulp each, far inside the 8-bit mantissa of the
-// result); fp32/fp64 storage uses libm and ATen's expression as written.
+// result); the exact form uses an erfc polynomial for 16-bit storage (see below);
+// fp32/fp64 storage uses libm and ATen's expression as written.
 #include "common.cuh"
 
 #include <math.h>
@@ -103,7 +104,39 @@ __device__ __forceinline__ float gelu_tanh_bwd_fast(float dy, float x) {
   return dy * (s * (1.0f + x * (1.0f - s) * inner_d2));
 }
 
-enum { kStoreWide = 0, kStoreNarrow = 1 };
+// Exact (erf) form for 16-bit data.  libm's erff costs more VALU time than the memory
+// traffic of a 16-bit element, so the normal CDF is formed from the complementary error
+// function in the Abramowitz-Stegun 7.1.26 shape
+//   erfc(z) = t (a1 + t (a2 + t (a3 + t (a4 + t a5)))) exp(-z^2),  t = 1 / (1 + p z),  z >= 0,
+// whose error is itself proportional to exp(-z^2): the relative error of erfc stays near
+// 1e-6 over the whole range, so Phi(x) = erfc(-x / sqrt 2) / 2 keeps full relative accuracy in
+// the left tail, where 1 + erf(.) cancels.  Far inside the 2^-9 / 2^-11 of a bf16 / f16 result.
+struct ErfcParts {
+  float half_erfc;  // erfc(|x| / sqrt 2) / 2
+  float gauss;      // exp(-x^2 / 2)
+};
+__device__ __forceinline__ ErfcParts half_erfc_abs(float x) {
+  constexpr float P = 0.3275911f * (float)kAlpha;  // p z = p |x| / sqrt 2
+  constexpr float A1 = 0.5f * 0.254829592f, A2 = 0.5f * -0.284496736f, A3 = 0.5f * 1.421413741f,
+                  A4 = 0.5f * -1.453152027f, A5 = 0.5f * 1.061405429f;
+  const float ax = fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(1.0f + P * ax);
+  const float poly = t * (A1 + t * (A2 + t * (A3 + t * (A4 + t * A5))));
+  ErfcParts r;
+  r.gauss = __builtin_amdgcn_exp2f(x * x * (float)(-0.5 * kLog2e));
+  r.half_erfc = poly * r.gauss;
+  return r;
+}
+__device__ __forceinline__ float gelu_erf_fwd_fast(float x) {
+  const ErfcParts e = half_erfc_abs(x);
+  const float cdf = x < 0.f ? e.half_erfc : 1.0f - e.half_erfc;
+  return x * cdf;
+}
+__device__ __forceinline__ float gelu_erf_bwd_fast(float dy, float x) {
+  const ErfcParts e = half_erfc_abs(x);
+  const float cdf = x < 0.f ? e.half_erfc : 1.0f - e.half_erfc;
+  return dy * (cdf + x * (e.gauss * (float)kPdfScale));
+}
 
 template <typename T, int MODE>
 __device__ __forceinline__ typename Acc<T>::type fwd_one(typename Acc<T>::type x) {
@@ -114,7 +147,11 @@ __device__ __forceinline__ typename Acc<T>::type fwd_one(typename Acc<T>::type x
       return gelu_tanh_fwd(x);
     }
   } else {
-    return gelu_erf_fwd(x);
+    if constexpr (sizeof(T) == 2) {
+      return gelu_erf_fwd_fast(x);
+    } else {
+      return gelu_erf_fwd(x);
+    }
   }
 }
 template <typename T, int MODE>
@@ -127,7 +164,11 @@ __device__ __forceinline__ typename Acc<T>::type bwd_one(typename Acc<T>::type d
       return gelu_tanh_bwd(dy, x);
     }
   } else {
-    return gelu_erf_bwd(dy, x);
+    if constexpr (sizeof(T) == 2) {
+      return gelu_erf_bwd_fast(dy, x);
+    } else {
+      return gelu_erf_bwd(dy, x);
+    }
   }
 }
 
