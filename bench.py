@@ -42,6 +42,7 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # algorithmic bytes per fused-classifier call: read the class columns of the logits once and
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
+CE_ROWS_TRAFFIC_BYTES = 1_650_851_000  # measured with rocprofv3 --pmc, see profiles/
 
 
 def log(*a):
@@ -171,7 +172,21 @@ def per_op_table(args, torch, ops):
         lib.cs_stream_copy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), src.numel(), stream)
 
     def wanted(name):
-        return not only or any(name.startswith(o) for o in only)
+        return not only or name == "stream_copy" or any(name.startswith(o) for o in only)
+
+    copy_points = []  # (bytes moved, ms) of the plain copy, the practical ceiling at each size
+
+    def copy_ms_at(nbytes):
+        """Time a plain copy moving `nbytes` would take, interpolated between measured sizes."""
+        pts = sorted(copy_points)
+        if not pts:
+            return None
+        if nbytes <= pts[0][0]:
+            return pts[0][1]  # below the smallest size the launch floor dominates
+        for (b0, t0), (b1, t1) in zip(pts, pts[1:]):
+            if nbytes <= b1:
+                return t0 + (t1 - t0) * (nbytes - b0) / (b1 - b0)
+        return pts[-1][1] * nbytes / pts[-1][0]
 
     def add(name, config, nbytes, make_set, call):
         """make_set() builds one set of buffers; call(set) issues the op once."""
@@ -191,9 +206,17 @@ def per_op_table(args, torch, ops):
             "frac_cold": round(nbytes / cold_med / 1e6 / HBM_PEAK_GBPS, 4),
             "buffer_sets": n_cold,
         }
+        if name == "stream_copy":
+            copy_points.append((nbytes, cold_med))
+        else:
+            ceiling = copy_ms_at(nbytes)
+            if ceiling:
+                rec["copy_ms_same_bytes"] = round(ceiling, 5)
+                rec["frac_of_copy"] = round(ceiling / cold_med, 3)
         out.append(rec)
         log(f"[per-op] {name:28s} {config:34s} warm {warm_med*1e3:9.1f} us  cold {cold_med*1e3:9.1f} us  "
-            f"{rec['gbps_cold']:8.1f} GB/s  {rec['frac_cold']*100:5.1f}% of HBM peak")
+            f"{rec['gbps_cold']:8.1f} GB/s  {rec['frac_cold']*100:5.1f}% of HBM peak"
+            + (f"  {rec['frac_of_copy']*100:5.1f}% of a plain copy" if "frac_of_copy" in rec else ""))
         del sets
         torch.cuda.empty_cache()
 
@@ -280,6 +303,10 @@ def per_op_table(args, torch, ops):
                "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
                "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
                "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1}
+        ceiling = copy_ms_at(nbytes)
+        if ceiling:
+            rec["copy_ms_same_bytes"] = round(ceiling, 5)
+            rec["frac_of_copy"] = round(ceiling / med, 3)
         out.append(rec)
         log(f"[per-op] adamw_multi_tensor           {tag:34s} {med*1e3:9.1f} us  {rec['gbps_cold']:8.1f} GB/s  "
             f"{rec['frac_cold']*100:5.1f}% of HBM peak")
@@ -429,7 +456,10 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_ms_avg": round(head["rows_kernel_ms_avg"], 5),
             "kernel_ms_median": round(head["rows_kernel_ms_median"], 5),
-            "traffic": None,
+            # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+            # profiles/ce_rows_stream_kernel_hbm_traffic_pmc.txt (scaled by a plain copy's readings)
+            "traffic": CE_ROWS_TRAFFIC_BYTES,
+            "traffic_over_algorithmic": round(CE_ROWS_TRAFFIC_BYTES / CE_BYTES, 4),
         },
         "cpu_baseline": cpu,
         "per_op": table,

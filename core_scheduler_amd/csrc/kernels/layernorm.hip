@@ -83,6 +83,20 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 }
 
 constexpr int kLnThreads = 256;  // 4 waves
+// backward launch shape; the defaults are the measured best, the macros exist for tuning runs
+#ifndef CS_LN_BWD_THREADS
+#define CS_LN_BWD_THREADS 512
+#endif
+#ifndef CS_LN_BWD_MAX_BLOCKS
+#define CS_LN_BWD_MAX_BLOCKS 256
+#endif
+#ifndef CS_LN_BWD_ROWS_VPL2
+#define CS_LN_BWD_ROWS_VPL2 2
+#endif
+#ifndef CS_LN_BWD_ROWS_VPL4
+#define CS_LN_BWD_ROWS_VPL4 1
+#endif
+constexpr int kLnBwdThreads = CS_LN_BWD_THREADS;
 
 // ------------------------------------------------------------ fast forward
 // VPL: 16-byte x vectors per lane; R: rows a wave handles per step.  A wave
@@ -203,7 +217,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
 // Same walk as the forward kernel, with dy and x prefetched one step ahead.
 template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int R, bool HAS_DX,
           bool HAS_DP>
-__global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
+__global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
     const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
     float *__restrict__ partial, int64_t rows, int C) {
@@ -211,7 +225,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
   extern __shared__ float lds[];  // [waves per block][C]
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
-  constexpr int kWaves = kLnThreads / kWave;
+  constexpr int kWaves = kLnBwdThreads / kWave;
   const int64_t gw = (int64_t)blockIdx.x * kWaves + wave;
   const int64_t step = (int64_t)gridDim.x * kWaves * R;
   const int nvec = C / VN;
@@ -318,7 +332,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_rows_kernel(
         }
       }
       __syncthreads();
-      for (int c = threadIdx.x; c < C; c += kLnThreads) {
+      for (int c = threadIdx.x; c < C; c += kLnBwdThreads) {
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) s += lds[w * C + c];
@@ -484,11 +498,11 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
   if (per_lane <= 2) {
     p.vpl = 2;
     p.fwd_rows = 4;
-    p.bwd_rows = 2;
+    p.bwd_rows = CS_LN_BWD_ROWS_VPL2;
   } else if (per_lane <= 4) {
     p.vpl = 4;
     p.fwd_rows = 2;
-    p.bwd_rows = 1;
+    p.bwd_rows = CS_LN_BWD_ROWS_VPL4;
   } else if (per_lane <= 8) {
     p.vpl = 8;
     p.fwd_rows = 1;
@@ -501,10 +515,10 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
 // the grid growing, which keeps the parameters in registers for many rows
 // and bounds the number of partial rows the backward pass leaves behind.
 constexpr int kLnFwdMaxBlocks = 1024;
-constexpr int kLnBwdMaxBlocks = 512;
+constexpr int kLnBwdMaxBlocks = CS_LN_BWD_MAX_BLOCKS;
 
-int ln_blocks(int64_t rows, int rows_per_wave, int cap) {
-  const int64_t rows_per_block = (int64_t)(kLnThreads / kWave) * rows_per_wave;
+int ln_blocks(int64_t rows, int rows_per_wave, int cap, int threads = kLnThreads) {
+  const int64_t rows_per_block = (int64_t)(threads / kWave) * rows_per_wave;
   const int64_t b = ceil_div(rows, rows_per_block);
   return (int)(b < cap ? b : cap);
 }
@@ -548,11 +562,11 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
-      const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks);
+      const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks, kLnBwdThreads);
       const size_t need = want_dp ? (size_t)blocks * 2 * C * sizeof(float) : 0;
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
-      const size_t lds = want_dp ? (size_t)(kLnThreads / kWave) * C * sizeof(float) : 0;
-      const dim3 grid((unsigned)blocks), block(kLnThreads);
+      const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
+      const dim3 grid((unsigned)blocks), block(kLnBwdThreads);
 #define CS_LN_BWD(VPL, R, HAS_DX, HAS_DP)                                                   \
   ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, R, HAS_DX, HAS_DP><<<grid, block, lds, s>>>(    \
       (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd,             \
@@ -566,9 +580,9 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
     CS_LN_BWD(VPL, R, false, true);           \
   }
       if (p.vpl == 2) {
-        CS_LN_BWD_MASK(2, 2)
+        CS_LN_BWD_MASK(2, CS_LN_BWD_ROWS_VPL2)
       } else if (p.vpl == 4) {
-        CS_LN_BWD_MASK(4, 1)
+        CS_LN_BWD_MASK(4, CS_LN_BWD_ROWS_VPL4)
       } else {
         CS_LN_BWD_MASK(8, 1)
       }
@@ -649,7 +663,7 @@ extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
   // the fast path's largest grid: one row per wave per step
-  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks) * 2 * (size_t)C * sizeof(float);
+  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads) * 2 * (size_t)C * sizeof(float);
 }
 
 extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
