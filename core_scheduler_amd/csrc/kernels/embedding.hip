@@ -13,25 +13,23 @@
 // independent of scheduling.  Four launches:
 //   1. tile sort  - each workgroup bitonic-sorts 1024 keys, one per lane:
 //                   exchanges below 64 lanes are wave shuffles, the rest go
-//                   through LDS.  Spare workgroups of the same launch clear
-//                   the row bitmap and sum the position-table gradient, which
-//                   needs no order.
+//                   through LDS.  Spare workgroups of the same launch sum the
+//                   position-table gradient, which needs no order.
 //   2. merge rank - every key finds its global rank by binary search in the
-//                   other tiles (staged in LDS), is scattered to its place,
-//                   and the first key of every id marks its row in a bitmap.
-//   3. reduce     - a segmented sum.  A workgroup owns 64 consecutive sorted
-//                   entries, each of its 16 waves owns 4 of them and loads
+//                   other tiles (staged in LDS) and is scattered to its place.
+//                   Launches 1 and 2 keep few CUs busy, so further workgroups
+//                   of both zero the whole table meanwhile (`=` semantics).
+//   3. reduce     - a segmented sum.  A workgroup owns 32 consecutive sorted
+//                   entries, each of its 8 waves owns 4 of them and loads
 //                   their rows at once.  Runs of equal ids inside a wave are
 //                   added in registers; runs that cross waves are folded
 //                   through LDS in wave order; a segment that crosses
 //                   workgroups leaves one fp32 partial row per workgroup, so
 //                   a hot row is read by as many CUs as it has windows.
-//                   Further workgroups of the same launch zero the rows
-//                   whose bitmap bit is clear.
 //   4. finish     - the workgroup of a crossing segment's first window adds
 //                   that segment's partial rows in window order.
-// The traffic that matters is the dense write of dweight (V*C elements) and
-// one read of dout.
+// The traffic that matters is the dense write of dweight (V*C elements), one
+// read of dout and a second write of the indexed rows.
 #include "common.cuh"
 
 #include <type_traits>
@@ -139,7 +137,10 @@ struct KeyCodec<uint64_t> {
 
 constexpr int kTile = 1024;  // keys per sorted tile = lanes of the sorting workgroup
 constexpr uint32_t kNoId = 0xFFFFFFFFu;
-constexpr int kWindow = 64;  // sorted entries per reducing workgroup
+#ifndef CS_EMB_WINDOW
+#define CS_EMB_WINDOW 32
+#endif
+constexpr int kWindow = CS_EMB_WINDOW;  // sorted entries per reducing workgroup (at most 64)
 
 // Position-table gradient for one 16-byte vector: dwpe[t, :] (+)= sum_b dout[b, t, :].
 template <typename T>
@@ -173,26 +174,50 @@ __device__ __forceinline__ void positions_vector(const T *__restrict__ dout, T *
   store16_stream(dwpe + f * VN, o);
 }
 
+// Zero fill of the table, spread over the sort and merge launches, whose own work leaves
+// most CUs idle.  Every row is zeroed before the reduce launch writes the indexed ones.
+// One fill workgroup clears kFillVecs 16-byte vectors.
+constexpr int kFillVecs = 8192;  // 128 KB
+#ifndef CS_EMB_FILL_SORT_PCT
+#define CS_EMB_FILL_SORT_PCT 40  // share of the table cleared in the sort launch
+#endif
+
+template <int THREADS>
+__device__ __forceinline__ void zero_fill_block(u32x4 *__restrict__ dst, int64_t vecs, int64_t blk,
+                                                int tid) {
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  const int64_t v0 = blk * kFillVecs;
+#pragma unroll 8
+  for (int u = 0; u < kFillVecs / THREADS; ++u) {
+    const int64_t i = v0 + (int64_t)u * THREADS + tid;
+    if (i < vecs) __builtin_nontemporal_store(z, dst + i);
+  }
+}
+
 // Launch layout, in block order:
 //   [0, n_tiles)                sort one tile of 1024 keys
-//   + 1                         preset sorted_id to "no id", clear the row bitmap
+//   + 1                         preset sorted_id to "no id"
 //   + pos_blocks                position-table gradient, 1024 vectors per block
+//   + the rest                  zero fill of fill_dst[0, fill_vecs)
 template <typename KeyT, typename IdxT, typename T>
 __global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
-    const IdxT *__restrict__ ids, KeyT *__restrict__ tiles, uint32_t *__restrict__ bitmap,
-    int64_t bitmap_words, uint32_t *__restrict__ sorted_id, int64_t n, int n_tiles, int shift,
-    int64_t num_weights, int64_t padding_idx, const T *__restrict__ dout, T *__restrict__ dwpe,
-    int64_t B, int64_t TC, int accumulate) {
+    const IdxT *__restrict__ ids, KeyT *__restrict__ tiles, uint32_t *__restrict__ sorted_id,
+    int64_t n, int n_tiles, int shift, int64_t num_weights, int64_t padding_idx,
+    const T *__restrict__ dout, T *__restrict__ dwpe, int64_t B, int64_t TC, int accumulate,
+    int64_t pos_blocks, u32x4 *__restrict__ fill_dst, int64_t fill_vecs) {
   __shared__ KeyT keys[2][kTile];
   const int tid = threadIdx.x;
   const int64_t blk = blockIdx.x;
+  if (blk > n_tiles + pos_blocks) {
+    zero_fill_block<kTile>(fill_dst, fill_vecs, blk - n_tiles - pos_blocks - 1, tid);
+    return;
+  }
   if (blk > n_tiles) {
     const int64_t f = (blk - n_tiles - 1) * kTile + tid;
     if (f < TC / Vec16<T>::n) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
     return;
   }
   if (blk == n_tiles) {
-    for (int64_t i = tid; i < bitmap_words; i += kTile) bitmap[i] = 0u;
     for (int64_t i = tid; i < n; i += kTile) sorted_id[i] = kNoId;
     return;
   }
@@ -231,14 +256,21 @@ __global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
 // them are searched side by side, so the probes overlap.
 constexpr int kMergeChunkBytes = 32768;
 
+// Blocks past the keys zero fill_dst[0, fill_vecs).
 template <typename KeyT>
 __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
-    const KeyT *__restrict__ tiles, uint32_t *__restrict__ bitmap,
-    uint32_t *__restrict__ sorted_id, uint32_t *__restrict__ sorted_pos, int n_tiles, int shift) {
+    const KeyT *__restrict__ tiles, uint32_t *__restrict__ sorted_id,
+    uint32_t *__restrict__ sorted_pos, int n_tiles, int shift, u32x4 *__restrict__ fill_dst,
+    int64_t fill_vecs) {
   constexpr int kChunkTiles = kMergeChunkBytes / (kTile * (int)sizeof(KeyT));
   constexpr int kSide = 4;
   constexpr int kVecPerThread = kMergeChunkBytes / 16 / kThreads;  // 8
   __shared__ u32x4 staged_raw[kMergeChunkBytes / 16];
+  const int64_t key_blocks = (int64_t)n_tiles * (kTile / kThreads);
+  if ((int64_t)blockIdx.x >= key_blocks) {
+    zero_fill_block<kThreads>(fill_dst, fill_vecs, (int64_t)blockIdx.x - key_blocks, threadIdx.x);
+    return;
+  }
   const KeyT *staged = reinterpret_cast<const KeyT *>(staged_raw);
   const int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const int own = (int)(g / kTile);  // block-uniform: 256 divides 1024
@@ -246,9 +278,6 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
   const KeyT key = tiles[g];
   const bool real = key != KeyCodec<KeyT>::kSentinel;
   int64_t rank = local;
-  // the global predecessor is the largest of the per-tile predecessors
-  bool has_pred = local > 0;
-  KeyT pred = has_pred ? tiles[g - 1] : (KeyT)0;
   for (int c0 = 0; c0 < n_tiles; c0 += kChunkTiles) {
     const int c_tiles = n_tiles - c0 < kChunkTiles ? n_tiles - c0 : kChunkTiles;
     const int c_vecs = c_tiles * kTile * (int)sizeof(KeyT) / 16;
@@ -287,72 +316,48 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
       for (int u = 0; u < kSide; ++u) {
         const int b = c0 + b0 + u;
         if (b0 + u >= c_tiles || b == own) continue;
-        // lb counts the keys < key so far; the key just below the bound is the tile's predecessor
+        // lb counts the keys < key so far; one last probe decides the element at the bound
         const KeyT at = tile[u][lb[u]];
-        const int count = lb[u] + (at < key ? 1 : 0);
-        rank += count;
-        if (count > 0) {
-          const KeyT cand = tile[u][count - 1];
-          if (!has_pred || cand > pred) pred = cand;
-          has_pred = true;
-        }
+        rank += lb[u] + (at < key ? 1 : 0);
       }
     }
   }
   if (!real) return;
-  const uint32_t id = KeyCodec<KeyT>::id(key, shift);
-  sorted_id[rank] = id;
+  sorted_id[rank] = KeyCodec<KeyT>::id(key, shift);
   sorted_pos[rank] = KeyCodec<KeyT>::pos(key, shift);
-  // the first key of an id marks the row as touched
-  if (!has_pred || KeyCodec<KeyT>::id(pred, shift) != id) atomicOr(&bitmap[id >> 5], 1u << (id & 31));
 }
 
 // ------------------------------------------------------ backward: reduction
-constexpr int kRedThreads = 1024;
-constexpr int kRedWaves = kRedThreads / kWave;  // 16
-constexpr int kOwn = kWindow / kRedWaves;       // 4 sorted entries per wave
+constexpr int kOwn = 4;                         // sorted entries per wave
+constexpr int kRedWaves = kWindow / kOwn;       // 8
+constexpr int kRedThreads = kRedWaves * kWave;  // 512: two workgroups share a CU
+constexpr int kFinThreads = 1024;               // finish kernel
+constexpr int kFinWaves = kFinThreads / kWave;
 constexpr int kVpl = 2;                         // 16-byte column vectors per lane per column chunk
 
-// Workgroup w reduces sorted entries [64 w, 64 w + 64).  partial rows live at
+// Workgroup w reduces sorted entries [kWindow w, kWindow (w + 1)).  partial rows live at
 // partial[(w*2 + slot) * C]: slot 0 for a run that came in over the window's
 // left edge and ends inside, slot 1 for a run that leaves over its right edge.
-constexpr int kFillRows = 64;  // rows per zero-fill workgroup
-
-// Launch layout: [0, n_windows) reduce one window each; the rest zero 64 rows each.
 template <typename T>
-__global__ __launch_bounds__(kRedThreads) void emb_bwd_reduce_kernel(
+__global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduce_kernel(
     const T *__restrict__ dout, const uint32_t *__restrict__ sorted_id,
-    const uint32_t *__restrict__ sorted_pos, const uint32_t *__restrict__ bitmap,
-    T *__restrict__ dweight, float *__restrict__ partial, int64_t n, int64_t C,
-    int64_t num_weights, int64_t n_windows, int accumulate) {
+    const uint32_t *__restrict__ sorted_pos, T *__restrict__ dweight, float *__restrict__ partial,
+    int64_t n, int64_t C, int accumulate) {
   constexpr int VN = Vec16<T>::n;
   constexpr int kChunkCols = kWave * kVpl * VN;
-  extern __shared__ float lds[];  // [16 waves][2 slots][kChunkCols]
+  extern __shared__ float lds[];  // [kRedWaves][2 slots][kChunkCols]
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int nvec = (int)(C / VN);
-  if ((int64_t)blockIdx.x >= n_windows) {
-    // ---- zero fill of rows nobody indexed; wave w takes rows w, w + 16, ... of this block's 64
-    const int64_t row0 = ((int64_t)blockIdx.x - n_windows) * kFillRows;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int r = 0; r < kFillRows / kRedWaves; ++r) {
-      const int64_t row = row0 + wave + (int64_t)r * kRedWaves;
-      if (row >= num_weights) break;
-      if ((bitmap[row >> 5] >> (row & 31)) & 1u) continue;  // wave-uniform
-      u32x4 *dst = reinterpret_cast<u32x4 *>(dweight + row * C);
-      for (int idx = lane; idx < nvec; idx += kWave) __builtin_nontemporal_store(z, dst + idx);
-    }
-    return;
-  }
   const int64_t w = blockIdx.x;
   const int64_t p0 = w * kWindow;
 
   // ---- ids of the window (lane l <-> entry p0 + l), the entry before and the entry after
   const int64_t p = p0 + lane;
-  const uint32_t my_id = p < n ? sorted_id[p] : kNoId;
-  const uint32_t prev_id = (p > 0 && p <= n) ? sorted_id[p - 1] : kNoId;
+  const bool in_window = lane < kWindow;
+  const uint32_t my_id = (in_window && p < n) ? sorted_id[p] : kNoId;
+  const uint32_t prev_id = (in_window && p > 0 && p <= n) ? sorted_id[p - 1] : kNoId;
   const uint64_t valid = __ballot(my_id != kNoId);
   if (valid == 0) return;  // nothing sorted into this window
   const int n_valid = __popcll(valid);  // valid entries are a prefix of the window
@@ -459,39 +464,55 @@ __global__ __launch_bounds__(kRedThreads) void emb_bwd_reduce_kernel(
       }
     }
     __syncthreads();
-    // ---- level 2: runs of the window that span waves, folded in wave order
+    // ---- level 2: runs of the window that span waves, folded in wave order.  A run that
+    // spans waves is folded by the wave it starts in (wave 0 for the run that came in over the
+    // left edge): that is at most one run per wave, so all folds proceed side by side.
     {
-      // a run spans waves exactly when some wave's first entry (4, 8, ... 60) is valid and is
-      // not a run start; walk those entries and fold each run once
-      uint64_t cont = ~starts & valid & 0x1111111111111110ull;
-      int prev_a = -1;
-      while (cont) {
-        const int q = __ffsll((long long)cont) - 1;
-        cont &= cont - 1;
-        const int a = 63 - __clzll((long long)(starts & ((1ull << q) - 1ull)));  // its run's start
-        if (a == prev_a) continue;
-        prev_a = a;
+      const int first = wave * kOwn;
+      const uint64_t mine = (starts >> first) & ((1ull << kOwn) - 1ull);  // run starts among my entries
+      const int boundary = first + kOwn;  // the next wave's first entry
+      const bool crosses = boundary < kWindow && ((valid >> boundary) & 1ull) &&
+                           !((starts >> boundary) & 1ull);
+      if (mine != 0 && crosses) {  // wave-uniform
+        const int a = first + (63 - __clzll((long long)mine));  // my last run start: the run that crosses
         const int b = run_end(a);
-        const int wa = a / kOwn, wb = (b - 1) / kOwn;
-        const int c = tid;       // one column of the chunk per thread
-        const int64_t col = (int64_t)cb * VN + c;
-        // read the id while every lane is still active: a shuffle cannot read an idle lane
+        const int wb = (b - 1) / kOwn;
+        const bool last_reaches_end = (b % kOwn) == 0;  // the run's piece in wave wb ends at its last entry
         const uint32_t id = __shfl(my_id, a, kWave);
-        if (c < kChunkCols && col < C) {
-          float t = 0.f;
-          for (int ww = wa; ww <= wb; ++ww) {
-            // wave ww's piece of this run reaches its last entry unless the run ends inside it
-            const int slot = (ww < wb || (b % kOwn) == 0) ? 1 : 0;
-            t += lds[(ww * 2 + slot) * kChunkCols + c];
-          }
-          const bool seg_begins = (heads >> a) & 1ull;
-          const bool seg_ends = !(b >= n_valid && leaves);
-          if (seg_begins && seg_ends) {
-            T *dst = dweight + (int64_t)id * C;
-            if (accumulate) t += to_acc(dst[col]);
-            dst[col] = from_acc<T>(t);
+        const bool seg_begins = (heads >> a) & 1ull;
+        const bool seg_ends = !(b >= n_valid && leaves);
+        const bool whole = seg_begins && seg_ends;
+        T *drow = dweight + (int64_t)id * C;
+        float *prow = partial + (w * 2 + (seg_ends ? 0 : 1)) * C;
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        const f32x4 *lds4 = reinterpret_cast<const f32x4 *>(lds);
+        constexpr int kSlices = kChunkCols / 4 / kWave;  // groups of four columns per lane
+        f32x4 t[kSlices];
+#pragma unroll
+        for (int v = 0; v < kSlices; ++v) t[v] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ww = wave; ww <= wb; ++ww) {
+          // wave ww's piece of this run reaches its last entry unless the run ends inside it
+          const int slot = (ww < wb || last_reaches_end) ? 1 : 0;
+          const f32x4 *src = lds4 + (ww * 2 + slot) * (kChunkCols / 4) + lane;
+          f32x4 x[kSlices];
+#pragma unroll
+          for (int v = 0; v < kSlices; ++v) x[v] = src[kWave * v];  // independent LDS reads
+#pragma unroll
+          for (int v = 0; v < kSlices; ++v) t[v] += x[v];
+        }
+#pragma unroll
+        for (int v = 0; v < kSlices; ++v) {
+          const int64_t col = (int64_t)cb * VN + (int64_t)(lane + kWave * v) * 4;
+          if (col >= C) continue;  // C is a multiple of four columns here
+          if (whole) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              float o = t[v][k];
+              if (accumulate) o += to_acc(drow[col + k]);
+              drow[col + k] = from_acc<T>(o);
+            }
           } else {
-            partial[(w * 2 + (seg_ends ? 0 : 1)) * C + col] = t;
+            *reinterpret_cast<f32x4 *>(prow + col) = t[v];
           }
         }
       }
@@ -507,10 +528,10 @@ __global__ __launch_bounds__(kRedThreads) void emb_bwd_reduce_kernel(
 // partial rows in window order: slot 1 of every window the segment leaves,
 // slot 0 of the one it ends in.
 template <typename T>
-__global__ __launch_bounds__(kRedThreads) void emb_bwd_finish_kernel(
+__global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
     const uint32_t *__restrict__ sorted_id, const float *__restrict__ partial,
     T *__restrict__ dweight, int64_t n, int64_t C, int accumulate) {
-  __shared__ int first_other[kRedWaves];
+  __shared__ int first_other[kFinWaves];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
@@ -524,14 +545,14 @@ __global__ __launch_bounds__(kRedThreads) void emb_bwd_finish_kernel(
   // windows after w whose last entry still has this id are left by the segment too; lane t
   // probes window w + 1 + t, 1024 windows per round
   int64_t w_hi = -1;  // the window the segment ends in
-  for (int64_t base = w + 1; w_hi < 0; base += kRedThreads) {
+  for (int64_t base = w + 1; w_hi < 0; base += kFinThreads) {
     const int64_t ww = base + tid;
     const int64_t q = ww * kWindow + kWindow - 1;
     const bool other = q >= n || sorted_id[q] != id;
     const uint64_t m = __ballot(other);
     if (lane == 0) first_other[wave] = m ? __ffsll((long long)m) - 1 : -1;
     __syncthreads();
-    for (int k = 0; k < kRedWaves; ++k) {
+    for (int k = 0; k < kFinWaves; ++k) {
       if (first_other[k] >= 0) {
         w_hi = base + k * kWave + first_other[k];
         break;
@@ -544,21 +565,29 @@ __global__ __launch_bounds__(kRedThreads) void emb_bwd_finish_kernel(
   const bool tail = w_hi * kWindow < n && sorted_id[w_hi * kWindow] == id;
   const int64_t w_end = tail ? w_hi : w_hi - 1;  // the window the segment ends in (> w)
   T *dst = dweight + (int64_t)id * C;
-  for (int64_t col = tid; col < C; col += kRedThreads) {
-    float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+  for (int64_t col = tid; col < C; col += kFinThreads) {
+    // eight interleaved sums keep eight loads in flight; the order is fixed all the same
+    float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     int64_t ww = w;
     // every window before the last is left over its right edge (slot 1)
-    for (; ww + 4 <= w_end; ww += 4) {
-      t0 += partial[((ww + 0) * 2 + 1) * C + col];
-      t1 += partial[((ww + 1) * 2 + 1) * C + col];
-      t2 += partial[((ww + 2) * 2 + 1) * C + col];
-      t3 += partial[((ww + 3) * 2 + 1) * C + col];
+    for (; ww + 8 <= w_end; ww += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = partial[((ww + u) * 2 + 1) * C + col];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] += v[u];
     }
-    for (; ww < w_end; ++ww) t0 += partial[(ww * 2 + 1) * C + col];
-    t1 += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
-    float t = (t0 + t1) + (t2 + t3);
-    if (accumulate) t += to_acc(dst[col]);
-    dst[col] = from_acc<T>(t);
+    {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = ww + u < w_end ? partial[((ww + u) * 2 + 1) * C + col] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 7; ++u) t[u] += v[u];  // at most seven windows are left
+    }
+    t[7] += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
+    float total = ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+    if (accumulate) total += to_acc(dst[col]);
+    dst[col] = from_acc<T>(total);
   }
 }
 
@@ -611,8 +640,7 @@ struct BwdLayout {
   bool key64 = false;
   int64_t n_tiles = 0;
   int64_t n_windows = 0;
-  int64_t bitmap_words = 0;
-  size_t off_bitmap = 0, off_tiles = 0, off_sorted_id = 0, off_sorted_pos = 0, off_partial = 0;
+  size_t off_tiles = 0, off_sorted_id = 0, off_sorted_pos = 0, off_partial = 0;
   size_t bytes = 0;
 };
 
@@ -626,10 +654,7 @@ BwdLayout bwd_layout(int64_t n, int64_t C, int64_t num_weights) {
   // ((V-1) << shift) | (2^shift - 1) must stay below the 32-bit sentinel
   L.key64 = L.shift >= 32 || ((uint64_t)num_weights << L.shift) > 0xFFFFFFFFull;
   L.n_windows = ceil_div(n, (int64_t)kWindow);
-  L.bitmap_words = ceil_div(num_weights, (int64_t)32);
   size_t o = 0;
-  L.off_bitmap = o;
-  o = align256(o + (size_t)L.bitmap_words * 4);
   L.off_tiles = o;
   o = align256(o + (size_t)padded * (L.key64 ? 8 : 4));
   L.off_sorted_id = o;
@@ -702,31 +727,37 @@ int fwd_dispatch(const void *weight, const void *wpe, const void *ids, void *out
   return CS_ERR_UNSUPPORTED;
 }
 
-// Sort + merge.  The sort launch also sums dwpe (`fused_positions`) on the CUs the sort
-// leaves idle.
+// Sort + merge.  The sort launch also sums dwpe (`fused_positions`), and both launches clear
+// their share of fill_dst[0, fill_vecs), on the CUs the sorting leaves idle.
 template <typename KeyT, typename IdxT, typename T>
 int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_t num_weights,
                 int64_t padding_idx, const T *dout, T *dwpe, bool fused_positions, int64_t B,
-                int64_t TC, int accumulate, hipStream_t s) {
+                int64_t TC, int accumulate, u32x4 *fill_dst, int64_t fill_vecs, hipStream_t s) {
   KeyT *tiles = reinterpret_cast<KeyT *>(ws + L.off_tiles);
-  uint32_t *bitmap = reinterpret_cast<uint32_t *>(ws + L.off_bitmap);
   uint32_t *sorted_id = reinterpret_cast<uint32_t *>(ws + L.off_sorted_id);
   uint32_t *sorted_pos = reinterpret_cast<uint32_t *>(ws + L.off_sorted_pos);
   const int64_t pos_blocks = fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)kTile) : 0;
-  const int64_t blocks = L.n_tiles + 1 + pos_blocks;
-  if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  // whole fill workgroups to the sort launch, the remainder to the merge launch
+  const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecs);
+  const int64_t sort_fill_blocks = fill_blocks * CS_EMB_FILL_SORT_PCT / 100;
+  const int64_t sort_fill_vecs =
+      sort_fill_blocks * kFillVecs < fill_vecs ? sort_fill_blocks * kFillVecs : fill_vecs;
+  const int64_t merge_fill_blocks = fill_blocks - sort_fill_blocks;
+  const int64_t blocks = L.n_tiles + 1 + pos_blocks + sort_fill_blocks;
+  const int64_t mblocks = L.n_tiles * kTile / kThreads + merge_fill_blocks;
+  if (blocks > 0x7fffffffLL || mblocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
   emb_bwd_tile_sort_kernel<KeyT, IdxT, T><<<dim3((unsigned)blocks), dim3(kTile), 0, s>>>(
-      (const IdxT *)ids, tiles, bitmap, L.bitmap_words, sorted_id, n, (int)L.n_tiles, L.shift,
-      num_weights, padding_idx, dout, dwpe, B, TC, accumulate);
+      (const IdxT *)ids, tiles, sorted_id, n, (int)L.n_tiles, L.shift, num_weights, padding_idx,
+      dout, dwpe, B, TC, accumulate, pos_blocks, fill_dst, sort_fill_vecs);
   int st = launch_status();
   if (st != CS_OK) return st;
-  const int64_t mblocks = L.n_tiles * kTile / kThreads;
   emb_bwd_merge_kernel<KeyT><<<dim3((unsigned)mblocks), dim3(kThreads), 0, s>>>(
-      tiles, bitmap, sorted_id, sorted_pos, (int)L.n_tiles, L.shift);
+      tiles, sorted_id, sorted_pos, (int)L.n_tiles, L.shift,
+      fill_dst ? fill_dst + sort_fill_vecs : nullptr, fill_vecs - sort_fill_vecs);
   return launch_status();
 }
 
-// The reduce kernel asks for 128 KB of LDS, above the 64 KB a launch gets by default.
+// The reduce kernel's dynamic LDS can exceed the 64 KB a launch gets by default (wide windows).
 template <typename T>
 int allow_reduce_lds(size_t bytes) {
   static bool done[64] = {false};
@@ -750,10 +781,13 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
                       is_aligned16(dweight) && (!dwpe || is_aligned16(dwpe));
   const bool fused_positions = vec_ok && dwpe != nullptr;
   const int64_t TC = T_len * C;
+  // `=` semantics on the fast path: the whole table is zeroed, then indexed rows are written
+  u32x4 *fill_dst = vec_ok && !accumulate ? reinterpret_cast<u32x4 *>(dweight) : nullptr;
+  const int64_t fill_vecs = fill_dst ? num_weights * (C / VN) : 0;
   int st;
 #define CS_SORT(KeyT, IdxT)                                                                      \
   sort_launch<KeyT, IdxT, T>(ids, ws, L, n, num_weights, padding_idx, (const T *)dout, (T *)dwpe, \
-                             fused_positions, B, TC, accumulate, s)
+                             fused_positions, B, TC, accumulate, fill_dst, fill_vecs, s)
   if (L.key64) {
     st = idx_dtype == CS_I64 ? CS_SORT(uint64_t, int64_t) : CS_SORT(uint64_t, int32_t);
   } else {
@@ -761,7 +795,6 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
   }
 #undef CS_SORT
   if (st != CS_OK) return st;
-  const uint32_t *bitmap = reinterpret_cast<const uint32_t *>(ws + L.off_bitmap);
   const uint32_t *sorted_id = reinterpret_cast<const uint32_t *>(ws + L.off_sorted_id);
   const uint32_t *sorted_pos = reinterpret_cast<const uint32_t *>(ws + L.off_sorted_pos);
   if (!vec_ok) {
@@ -779,19 +812,16 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
   if constexpr (!std::is_same_v<T, double>) {
     float *partial = reinterpret_cast<float *>(ws + L.off_partial);
     const int64_t windows = n > 0 ? L.n_windows : 0;
-    const int64_t fill_blocks = accumulate ? 0 : ceil_div(num_weights, (int64_t)kFillRows);
-    const int64_t blocks = windows + fill_blocks;
-    if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
-    if (blocks == 0) return CS_OK;
+    if (windows > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+    if (windows == 0) return CS_OK;
     const size_t lds = (size_t)kRedWaves * 2 * kWave * kVpl * VN * sizeof(float);
     st = allow_reduce_lds<T>(lds);
     if (st != CS_OK) return st;
-    emb_bwd_reduce_kernel<T><<<dim3((unsigned)blocks), dim3(kRedThreads), lds, s>>>(
-        (const T *)dout, sorted_id, sorted_pos, bitmap, (T *)dweight, partial, n, C, num_weights,
-        windows, accumulate);
+    emb_bwd_reduce_kernel<T><<<dim3((unsigned)windows), dim3(kRedThreads), lds, s>>>(
+        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, partial, n, C, accumulate);
     st = launch_status();
-    if (st != CS_OK || windows == 0) return st;
-    emb_bwd_finish_kernel<T><<<dim3((unsigned)windows), dim3(kRedThreads), 0, s>>>(
+    if (st != CS_OK) return st;
+    emb_bwd_finish_kernel<T><<<dim3((unsigned)windows), dim3(kFinThreads), 0, s>>>(
         sorted_id, partial, (T *)dweight, n, C, accumulate);
     return launch_status();
   }

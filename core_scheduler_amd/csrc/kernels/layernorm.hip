@@ -68,6 +68,17 @@ __device__ __forceinline__ Raw<T, N> load_raw(const T *p) {
   for (int q = 0; q < N / Vec16<T>::n; ++q) r.v[q] = load16_stream(p + q * Vec16<T>::n);
   return r;
 }
+// Makes the compiler forget what it derived from the packed values, so code after
+// this point unpacks them again instead of keeping the unpacked floats in registers.
+template <typename T, int N>
+__device__ __forceinline__ void forget_unpacked(Raw<T, N> &r) {
+#pragma unroll
+  for (int q = 0; q < N / Vec16<T>::n; ++q) {
+    u32x4 w = __builtin_bit_cast(u32x4, r.v[q]);
+    asm volatile("" : "+v"(w));
+    r.v[q] = __builtin_bit_cast(Vec16<T>, w);
+  }
+}
 template <typename T, int N>
 __device__ __forceinline__ Raw<T, N> zero_raw() {
   Raw<T, N> r;
@@ -274,36 +285,42 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
     for (int r = 0; r < R; ++r) {
       if (row0 + r >= rows) break;
       float s1 = 0.f, s2 = 0.f;
-      float xh[VPL][VN], dv[VPL][VN];
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
 #pragma unroll
         for (int k = 0; k < VN; ++k) {
           // lanes past the row hold zeros in dy, so they add nothing
-          xh[j][k] = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
-          dv[j][k] = raw_get<TDY, VN>(dcur.v[r][j], k);
+          const float xh = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
+          const float dv = raw_get<TDY, VN>(dcur.v[r][j], k);
           if constexpr (HAS_DP) {
-            acc_g[j][k] += dv[j][k] * xh[j][k];
-            acc_b[j][k] += dv[j][k];
+            acc_g[j][k] += dv * xh;
+            acc_b[j][k] += dv;
           }
           if constexpr (HAS_DX) {
-            const float gd = dv[j][k] * g[j][k];
+            const float gd = dv * g[j][k];
             s1 += gd;
-            s2 += gd * xh[j][k];
+            s2 += gd * xh;
           }
         }
       }
       if constexpr (HAS_DX) {
         s1 = wave_reduce(s1, SumOp{}) * inv_c;
         s2 = wave_reduce(s2, SumOp{}) * inv_c;
+        // x-hat and dy are unpacked again from the packed row rather than kept as
+        // floats across the reduction: half the registers, a few more VALU ops
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
+          forget_unpacked(xcur.v[r][j]);
+          forget_unpacked(dcur.v[r][j]);
           const int idx = lane + kWave * j;
           if (idx < nvec) {
             float o[VN];
 #pragma unroll
-            for (int k = 0; k < VN; ++k)
-              o[k] = rs[r] * (dv[j][k] * g[j][k] - s1 - xh[j][k] * s2);
+            for (int k = 0; k < VN; ++k) {
+              const float xh = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
+              const float dv = raw_get<TDY, VN>(dcur.v[r][j], k);
+              o[k] = rs[r] * (dv * g[j][k] - s1 - xh * s2);
+            }
             store_n<TDX, VN>(dx + (row0 + r) * C + (int64_t)idx * VN, o);
           }
         }
