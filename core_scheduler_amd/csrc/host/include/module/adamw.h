@@ -1,0 +1,28 @@
+// cs::module::AdamW (the reference's include/module/adamw.h:22-41).  step() updates every
+// parameter of the module tree; where the reference submits one task and one kernel launch
+// per parameter (src/module/adamw.cpp:32-38), this one submits one task with one launch for
+// each group of parameters that share dtype, hyper-parameters and step count: one launch for
+// a model built the usual way.
+#pragma once
+#include "module/optimizer_module.h"
+#include "module/pimpl.h"
+#include "optimizer/adamw.h"
+
+namespace cs::module {
+struct CS_API AdamWImpl : OptimizerModule {
+  using Options = optimizer::AdamW::Options;
+
+  explicit AdamWImpl(const Scheduler &scheduler, const Module &module, const Options &options);
+
+  template <typename ModuleHolder, typename = std::enable_if_t<!std::is_base_of_v<module::Module, ModuleHolder>>>
+  explicit AdamWImpl(const Scheduler &scheduler, const ModuleHolder &module, const Options &options)
+      : AdamWImpl{scheduler, *module, options} {}
+
+  void step(const Scheduler &scheduler) const override;
+
+ protected:
+  AdamWImpl() = default;
+};
+
+CS_MODULE(AdamW);
+}  // namespace cs::module

@@ -1,0 +1,60 @@
+// cs::module::Module: a tree of named submodules, each with at most one parameter state
+// (the reference's include/module/module.h:27-69, src/module/module.cpp:33-127).
+#pragma once
+#include <torch/nn/pimpl.h>
+
+#include <functional>
+#include <memory>
+#include <stdexcept>
+#include <string>
+
+#include "module/state.h"
+
+namespace cs::module {
+struct CS_API Module : std::enable_shared_from_this<Module> {
+  virtual ~Module() = default;
+  using NamedModulePointerApplyFunction = std::function<void(const std::string &, const std::shared_ptr<Module> &)>;
+  using ConstNamedModuleApplyFunction = std::function<void(const std::string &, const Module &)>;
+
+  // depth-first over the children, names joined with '.'
+  void apply_to_submodules(const NamedModulePointerApplyFunction &function,
+                           const std::string &name_prefix = std::string(), std::size_t depth = 0) const;
+  // this module first (under `name_prefix`), then every submodule
+  void apply(const ConstNamedModuleApplyFunction &function, const std::string &name_prefix = {}) const;
+
+  void register_state(std::shared_ptr<State> state);
+
+  template <typename ModuleType>
+  std::shared_ptr<ModuleType> register_module(std::string name, std::shared_ptr<ModuleType> module);
+  template <typename ModuleType>
+  std::shared_ptr<ModuleType> register_module(std::string name, torch::nn::ModuleHolder<ModuleType> module_holder);
+
+  OrderedDict<std::string, std::shared_ptr<State>> named_states() const;
+  // keys are "<module path>.<name inside the state>", e.g. "wte.weight"
+  OrderedDict<std::string, Tensor> named_parameters(bool recurse = true) const;
+  OrderedDict<std::string, Tensor> named_gradients(bool recurse = true) const;
+  OrderedDict<std::string, State::Increment> named_increments(bool recurse = true) const;
+
+  void zero_grad() const;  // gradients become undefined handles
+  void to(TensorOptions options) const;
+
+ protected:
+  OrderedDict<std::string, std::shared_ptr<Module>> children_;
+  std::shared_ptr<State> state_;
+};
+
+template <typename ModuleType>
+std::shared_ptr<ModuleType> Module::register_module(std::string name, std::shared_ptr<ModuleType> module) {
+  if (name.empty()) throw std::runtime_error("Submodule name must not be empty");
+  if (name.find('.') != std::string::npos)
+    throw std::runtime_error("Submodule name must not contain a dot (got '" + name + "')");
+  auto &base = children_.insert(std::move(name), std::move(module));
+  return std::dynamic_pointer_cast<ModuleType>(base);
+}
+
+template <typename ModuleType>
+std::shared_ptr<ModuleType> Module::register_module(std::string name,
+                                                    torch::nn::ModuleHolder<ModuleType> module_holder) {
+  return register_module(std::move(name), module_holder.ptr());
+}
+}  // namespace cs::module

@@ -1,0 +1,26 @@
+// cs::module::OptimizerModule: the optimizer states of every parameter of a module tree
+// (the reference's include/module/optimizer_module.h:29-52, src/module/optimizer_module.cpp:22-41).
+#pragma once
+#include <memory>
+#include <string>
+
+#include "module/module.h"
+#include "module/state.h"
+#include "threading/scheduler.h"
+
+namespace cs::module {
+struct CS_API OptimizerModule : std::enable_shared_from_this<OptimizerModule> {
+  virtual ~OptimizerModule() = default;
+
+  OrderedDict<std::string, std::shared_ptr<OptimizerState>> named_states() const;
+  void set_lr(double lr) const;
+  double get_lr() const;
+  virtual void step(const Scheduler &scheduler) const = 0;
+  // gradients are set to undefined, not to zero
+  void zero_grad(const Scheduler &scheduler) const;
+
+ protected:
+  OrderedDict<std::string, std::shared_ptr<OptimizerState>> states_;
+  std::weak_ptr<const Module> module_;
+};
+}  // namespace cs::module

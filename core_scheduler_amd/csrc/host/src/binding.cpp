@@ -14,6 +14,10 @@
 #include "compute/gelu.h"
 #include "compute/layer_norm.h"
 #include "memory/to_torch.h"
+#include "module/adamw.h"
+#include "module/embedding.h"
+#include "module/layer_norm.h"
+#include "module/module.h"
 #include "optimizer/adamw.h"
 #include "tensor_impl.h"
 #include "threading/dynamic_scheduler.h"
@@ -40,6 +44,14 @@ c10::DeviceIndex device_of(const Scheduler &s) {
 struct AutocastScope {
   std::unique_ptr<autocast::ContextGuard> guard;
 };
+// a module with no state of its own, to build trees from Python
+struct Container final : module::Module {};
+template <typename Value>
+std::vector<std::pair<std::string, Value>> items(const OrderedDict<std::string, Value> &dict) {
+  std::vector<std::pair<std::string, Value>> out;
+  for (const auto &kv : dict) out.emplace_back(kv.key(), kv.value());
+  return out;
+}
 }  // namespace
 
 PYBIND11_MODULE(_cs_host, m) {
@@ -173,5 +185,71 @@ PYBIND11_MODULE(_cs_host, m) {
       std::vector<ReadOnlyTensor> grads(dws.begin(), dws.end());
       Op::step(s, base, ws, grads);
     });
+  }
+  // ---- module layer
+  {
+    using module::Module;
+    py::class_<Module, std::shared_ptr<Module>>(m, "Module")
+        .def("named_parameters", [](const Module &mod) { return items(mod.named_parameters()); })
+        .def("named_gradients", [](const Module &mod) { return items(mod.named_gradients()); })
+        .def("named_states", [](const Module &mod) {
+          std::vector<std::string> names;
+          for (const auto &kv : mod.named_states()) names.push_back(kv.key());
+          return names;
+        })
+        .def("named_increments", [](const Module &mod) {
+          std::vector<std::tuple<std::string, Tensor, Tensor>> out;
+          for (const auto &kv : mod.named_increments())
+            out.emplace_back(kv.key(), kv.value().parameter, kv.value().gradient);
+          return out;
+        })
+        .def("zero_grad", &Module::zero_grad)
+        .def("to", [](const Module &mod, const std::string &dtype) { mod.to(at::TensorOptions().dtype(dtype_from(dtype))); });
+    py::class_<Container, Module, std::shared_ptr<Container>>(m, "Container")
+        .def(py::init([]() { return std::make_shared<Container>(); }))
+        .def("register_module", [](Container &c, const std::string &name, const std::shared_ptr<Module> &child) {
+          return c.register_module(name, child);
+        });
+    py::class_<module::EmbeddingImpl, Module, std::shared_ptr<module::EmbeddingImpl>>(m, "EmbeddingModule")
+        .def(py::init([](const Scheduler &s, int64_t n, int64_t d, const std::string &dtype) {
+               return std::make_shared<module::EmbeddingImpl>(
+                   s, module::EmbeddingImpl::Options{n, d}.device(at::Device(at::kCUDA, device_of(s))).dtype(dtype_from(dtype)));
+             }),
+             py::arg("scheduler"), py::arg("num_embeddings"), py::arg("embedding_dim"), py::arg("dtype") = "float32")
+        .def("forward", &module::EmbeddingImpl::forward)
+        .def("backward", &module::EmbeddingImpl::backward)
+        .def("state", &module::EmbeddingImpl::state);
+    py::class_<module::LayerNormImpl, Module, std::shared_ptr<module::LayerNormImpl>>(m, "LayerNormModule")
+        .def(py::init([](const Scheduler &s, std::vector<int64_t> shape, double eps, bool bias, const std::string &dtype) {
+               return std::make_shared<module::LayerNormImpl>(
+                   s, module::LayerNormImpl::Options{shape}.eps(eps).bias(bias)
+                          .device(at::Device(at::kCUDA, device_of(s))).dtype(dtype_from(dtype)));
+             }),
+             py::arg("scheduler"), py::arg("normalized_shape"), py::arg("eps") = 1e-5, py::arg("bias") = true,
+             py::arg("dtype") = "float32")
+        .def("forward", &module::LayerNormImpl::forward)
+        .def("backward", &module::LayerNormImpl::backward)
+        .def("state", &module::LayerNormImpl::state);
+    py::class_<module::AdamWImpl, std::shared_ptr<module::AdamWImpl>>(m, "AdamWModule")
+        .def(py::init([](const Scheduler &s, const std::shared_ptr<Module> &mod, double lr, double beta1, double beta2,
+                         double eps, double weight_decay, bool amsgrad, long t) {
+               return std::make_shared<module::AdamWImpl>(
+                   s, *mod,
+                   module::AdamWImpl::Options{}.lr(lr).beta1(beta1).beta2(beta2).eps(eps).weight_decay(weight_decay)
+                       .amsgrad(amsgrad).t(t));
+             }),
+             py::arg("scheduler"), py::arg("module"), py::arg("lr") = 1e-3, py::arg("beta1") = 0.9,
+             py::arg("beta2") = 0.999, py::arg("eps") = 1e-8, py::arg("weight_decay") = 1e-2,
+             py::arg("amsgrad") = false, py::arg("t") = 0)
+        .def("step", &module::AdamWImpl::step)
+        .def("zero_grad", &module::AdamWImpl::zero_grad)
+        .def("set_lr", &module::AdamWImpl::set_lr)
+        .def("get_lr", &module::AdamWImpl::get_lr)
+        .def("named_states", [](const module::AdamWImpl &o) {
+          std::vector<std::pair<std::string, std::shared_ptr<optimizer::AdamW::State>>> out;
+          for (const auto &kv : o.named_states())
+            out.emplace_back(kv.key(), std::dynamic_pointer_cast<optimizer::AdamW::State>(kv.value()));
+          return out;
+        });
   }
 }

@@ -268,6 +268,93 @@ def test_adamw_all_parameters_in_one_task(host, sched, co):
     assert_bit_exact(down(host, sched, ws[1]), before, "skipped update")
 
 
+# ------------------------------------------------------------------- module layer
+def build_tree(host, sched, V=211, T=16, C=64):
+    """A GPT-2-shaped tree: wte, wpe, h.0.ln_1, h.0.ln_2, ln_f (what the ops here cover)."""
+    root = host.Container()
+    wte = root.register_module("wte", host.EmbeddingModule(sched, V, C))
+    wpe = root.register_module("wpe", host.EmbeddingModule(sched, T, C))
+    h = root.register_module("h", host.Container())
+    block = h.register_module("0", host.Container())
+    ln1 = block.register_module("ln_1", host.LayerNormModule(sched, [C]))
+    ln2 = block.register_module("ln_2", host.LayerNormModule(sched, [C], bias=False))
+    lnf = root.register_module("ln_f", host.LayerNormModule(sched, [C]))
+    return root, dict(wte=wte, wpe=wpe, ln1=ln1, ln2=ln2, lnf=lnf)
+
+
+@pytest.mark.gpu
+def test_module_tree_names_and_zero_grad(host, sched):
+    # src/module/module.cpp:33-120: depth-first order, names joined with '.', state name appended
+    root, mods = build_tree(host, sched)
+    assert root.named_states() == ["wte", "wpe", "h.0.ln_1", "h.0.ln_2", "ln_f"]
+    names = [k for k, _ in root.named_parameters()]
+    assert names == ["wte.weight", "wpe.weight", "h.0.ln_1.weight", "h.0.ln_1.bias", "h.0.ln_2.weight",
+                     "ln_f.weight", "ln_f.bias"]
+    assert [k for k, _ in root.named_gradients()] == names
+    assert all(not g.defined() for _, g in root.named_gradients())  # nothing has run backward yet
+    B, T, C = 2, 16, 64
+    ids = randint(0, 211, (B, T), 5, dtype=torch.int64)
+    x = mods["wte"].forward(sched, up(host, sched, ids))
+    y = mods["ln1"].forward(sched, x)
+    dy = up(host, sched, randn((B, T, C), 6))
+    dx = mods["ln1"].backward(sched, dy)
+    mods["wte"].backward(sched, dx)
+    grads = dict(root.named_gradients())
+    for k in ("wte.weight", "h.0.ln_1.weight", "h.0.ln_1.bias"):
+        grads[k].wait()
+        assert grads[k].defined(), k
+    assert not grads["ln_f.weight"].defined()
+    root.zero_grad()  # set to undefined, as the reference does (src/compute/embedding.cpp:54)
+    assert all(not g.defined() for _, g in root.named_gradients())
+    root.to("bfloat16")
+    assert all(down(host, sched, p).dtype == torch.bfloat16 for _, p in root.named_parameters())
+
+
+@pytest.mark.gpu
+def test_adamw_module_matches_torch_optimizer(host, sched):
+    # test/test_adamw.cpp:105-190 checks cs::module::AdamW against torch::optim::AdamW on the same
+    # parameters and gradients with tolerance (1e-4, 1e-5); here over a tree and three steps.
+    # (amsgrad is left out: the reference keeps the maximum of the bias-corrected second moment,
+    # src/optimizer/adamw.cu:80-82, torch.optim the maximum of the raw one.)
+    amsgrad = False
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    root, mods = build_tree(host, sched)
+    opt = host.AdamWModule(sched, root, amsgrad=amsgrad, **hp)
+    names = [k for k, _ in root.named_parameters()]
+    assert [k for k, _ in opt.named_states()] == names
+    ref_params = {k: torch.nn.Parameter(down(host, sched, p).clone()) for k, p in root.named_parameters()}
+    ref = torch.optim.AdamW(ref_params.values(), lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"],
+                            weight_decay=hp["weight_decay"], amsgrad=amsgrad, foreach=False)
+    B, T, C = 2, 16, 64
+    for step in range(3):
+        ids = randint(0, 211, (B, T), 50 + step, dtype=torch.int64)
+        x = mods["wte"].forward(sched, up(host, sched, ids))
+        y = mods["ln1"].forward(sched, x)
+        z = mods["lnf"].forward(sched, y)
+        dz = up(host, sched, randn((B, T, C), 60 + step))
+        dy = mods["lnf"].backward(sched, dz)
+        dx = mods["ln1"].backward(sched, dy)
+        mods["wte"].backward(sched, dx)
+        grads = dict(root.named_gradients())
+        for k, p in ref_params.items():  # wpe and h.0.ln_2 were not used: no gradient, no update
+            p.grad = down(host, sched, grads[k]).clone() if k in ("wte.weight", "h.0.ln_1.weight", "h.0.ln_1.bias",
+                                                                 "ln_f.weight", "ln_f.bias") else None
+        opt.step(sched)
+        ref.step()
+        opt.zero_grad(sched)
+    for k, p in root.named_parameters():
+        got = down(host, sched, p)
+        assert torch.allclose(got, ref_params[k].detach(), 1e-4, 1e-5), k
+    states = dict(opt.named_states())
+    assert all(s.t == 3 for s in states.values())
+    assert torch.allclose(down(host, sched, states["wte.weight"].m), ref.state[ref_params["wte.weight"]]["exp_avg"],
+                          1e-4, 1e-6)
+    assert torch.allclose(down(host, sched, states["ln_f.bias"].v), ref.state[ref_params["ln_f.bias"]]["exp_avg_sq"],
+                          1e-4, 1e-9)
+    opt.set_lr(5e-3)
+    assert opt.get_lr() == 5e-3 and all(s.get_lr() == 5e-3 for s in states.values())
+
+
 # ------------------------------------------------------ error conventions (no GPU)
 def run_snippet(code):
     env = dict(os.environ, PYTHONPATH=ROOT)
@@ -296,3 +383,19 @@ def test_embedding_argument_checks_raise():
                 print("raised:", str(e).splitlines()[0])
     """)
     assert p.stdout.count("raised:") == 3, p.stdout + p.stderr
+
+
+def test_module_names_are_checked():
+    # include/module/module.h:73-85: empty names and names with a dot are rejected
+    p = run_snippet("""
+        from core_scheduler_amd import _cs_host as h
+        root = h.Container()
+        for name in ("", "a.b"):
+            try:
+                root.register_module(name, h.Container())
+            except RuntimeError as e:
+                print("raised:", e)
+        root.register_module("ok", h.Container())
+        print("states:", root.named_states(), "parameters:", root.named_parameters())
+    """)
+    assert p.stdout.count("raised:") == 2 and "states: [] parameters: []" in p.stdout, p.stdout + p.stderr
