@@ -311,6 +311,15 @@ def per_op_table(args, torch, ops):
         log(f"[per-op] adamw_multi_tensor           {tag:34s} {med*1e3:9.1f} us  {rec['gbps_cold']:8.1f} GB/s  "
             f"{rec['frac_cold']*100:5.1f}% of HBM peak")
         if tag == "small":
+            # global-norm clipping folded into the step: a 4 B/parameter norm pass, then the step
+            opt.step(max_grad_norm=1.0)
+            med_c, _ = event_ms(lambda i: opt.step(max_grad_norm=1.0), reps, torch)
+            nb_c = 32 * total
+            out.append({"op": "adamw_multi_tensor_clipped", "config": f"{tag} norm pass + step, {total} fp32 params",
+                        "algorithmic_bytes": nb_c, "ms_warm": round(med_c, 5), "ms_cold": round(med_c, 5),
+                        "gbps_warm": round(nb_c / med_c / 1e6, 1), "gbps_cold": round(nb_c / med_c / 1e6, 1),
+                        "frac_cold": round(nb_c / med_c / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1})
+            log(f"[per-op] adamw + grad-norm clip       {tag:34s} {med_c*1e3:9.1f} us  {nb_c / med_c / 1e6:8.1f} GB/s")
             # the reference's launch shape: one launch per tensor (src/module/adamw.cpp:32-38)
             ms_, vs_ = [torch.zeros_like(x) for x in ws_], [torch.zeros_like(x) for x in ws_]
 

@@ -50,6 +50,16 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_int] + [c_double] * 5 + [c_int64, c_void_p],
     ),
+    "cs_grad_norm_multi_workspace_bytes": (c_size_t, [c_int64]),
+    "cs_grad_norm_multi": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int, c_double, c_double, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p],
+    ),
+    "cs_grad_scale_multi": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p]),
+    "cs_adamw_multi_step_clipped": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int, c_int] + [c_double] * 5 + [c_int64, c_void_p, c_void_p],
+    ),
     "cs_gelu_forward": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "cs_gelu_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "cs_layernorm_forward": (

@@ -20,8 +20,14 @@ struct CS_API AdamWImpl : OptimizerModule {
 
   void step(const Scheduler &scheduler) const override;
 
+  // With Options::max_grad_norm set: the global gradient norm of the last step (an undefined
+  // handle before the first one).  Clipping needs all parameters in one launch group.
+  [[nodiscard]] Tensor last_grad_norm() const { return last_grad_norm_; }
+
  protected:
   AdamWImpl() = default;
+  c10::optional<double> max_grad_norm_{};
+  mutable Tensor last_grad_norm_{};
 };
 
 CS_MODULE(AdamW);

@@ -40,6 +40,10 @@ struct CS_API AdamW {
     CS_ARG(double, weight_decay) = 1e-2;
     CS_ARG(bool, amsgrad) = false;
     CS_ARG(long, t) = 0;
+    // Not in the reference (its example leaves clipping as a TODO,
+    // example/gpt2/gpt2_single_device.cpp:706): module::AdamW clips the global gradient norm to
+    // this value inside its step.
+    CS_ARG(c10::optional<double>, max_grad_norm) = {};
   };
 
   static std::shared_ptr<State> init(const Scheduler &scheduler, const ReadOnlyTensor &parameter,
@@ -55,5 +59,13 @@ struct CS_API AdamW {
   static void step(const Scheduler &scheduler,
                    const std::vector<std::shared_ptr<module::OptimizerState>> &states,
                    const std::vector<Tensor> &ws, const std::vector<ReadOnlyTensor> &dws);
+
+  // The same with Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746) folded in: the global
+  // norm is taken first and the step scales each gradient as it reads it, so the gradients
+  // themselves are left as they were.  Returns the 0-d norm (undefined handle if nothing ran).
+  static Tensor step(const Scheduler &scheduler,
+                     const std::vector<std::shared_ptr<module::OptimizerState>> &states,
+                     const std::vector<Tensor> &ws, const std::vector<ReadOnlyTensor> &dws,
+                     c10::optional<double> max_grad_norm, double norm_type = 2.0);
 };
 }  // namespace cs::optimizer

@@ -13,6 +13,7 @@
 #include "compute/embedding.h"
 #include "compute/gelu.h"
 #include "compute/layer_norm.h"
+#include "compute/utils.h"
 #include "memory/to_torch.h"
 #include "module/adamw.h"
 #include "module/embedding.h"
@@ -71,6 +72,8 @@ PYBIND11_MODULE(_cs_host, m) {
   py::class_<Tensor, ReadOnlyTensor>(m, "Tensor").def(py::init<>());
 
   m.def("to_torch", &memory::to_torch, py::arg("scheduler"), py::arg("tensor"));
+  m.def("clip_grad_norm_", &compute::Utils::clip_grad_norm_, py::arg("scheduler"), py::arg("tensors"),
+        py::arg("max_norm"), py::arg("norm_type") = 2.0);
   m.def("from_torch", &memory::from_torch, py::arg("scheduler"), py::arg("tensor"));
 
   py::class_<AutocastScope>(m, "autocast")
@@ -232,16 +235,17 @@ PYBIND11_MODULE(_cs_host, m) {
         .def("state", &module::LayerNormImpl::state);
     py::class_<module::AdamWImpl, std::shared_ptr<module::AdamWImpl>>(m, "AdamWModule")
         .def(py::init([](const Scheduler &s, const std::shared_ptr<Module> &mod, double lr, double beta1, double beta2,
-                         double eps, double weight_decay, bool amsgrad, long t) {
-               return std::make_shared<module::AdamWImpl>(
-                   s, *mod,
-                   module::AdamWImpl::Options{}.lr(lr).beta1(beta1).beta2(beta2).eps(eps).weight_decay(weight_decay)
-                       .amsgrad(amsgrad).t(t));
+                         double eps, double weight_decay, bool amsgrad, long t, std::optional<double> max_grad_norm) {
+               auto o = module::AdamWImpl::Options{}.lr(lr).beta1(beta1).beta2(beta2).eps(eps)
+                            .weight_decay(weight_decay).amsgrad(amsgrad).t(t);
+               if (max_grad_norm) o = o.max_grad_norm(*max_grad_norm);
+               return std::make_shared<module::AdamWImpl>(s, *mod, o);
              }),
              py::arg("scheduler"), py::arg("module"), py::arg("lr") = 1e-3, py::arg("beta1") = 0.9,
              py::arg("beta2") = 0.999, py::arg("eps") = 1e-8, py::arg("weight_decay") = 1e-2,
-             py::arg("amsgrad") = false, py::arg("t") = 0)
+             py::arg("amsgrad") = false, py::arg("t") = 0, py::arg("max_grad_norm") = py::none())
         .def("step", &module::AdamWImpl::step)
+        .def("last_grad_norm", &module::AdamWImpl::last_grad_norm)
         .def("zero_grad", &module::AdamWImpl::zero_grad)
         .def("set_lr", &module::AdamWImpl::set_lr)
         .def("get_lr", &module::AdamWImpl::get_lr)

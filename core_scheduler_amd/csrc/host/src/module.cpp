@@ -136,6 +136,7 @@ AdamWImpl::AdamWImpl(const Scheduler &scheduler, const Module &module, const Opt
   for (const auto &parameter : module.named_parameters())
     states_.insert(parameter.key(), optimizer::AdamW::init(scheduler, parameter.value(), options));
   module_ = module.weak_from_this();
+  max_grad_norm_ = options.max_grad_norm();
 }
 
 void AdamWImpl::step(const Scheduler &scheduler) const {
@@ -169,9 +170,12 @@ void AdamWImpl::step(const Scheduler &scheduler) const {
     found->second.parameters.push_back(increment->parameter);
     found->second.gradients.push_back(increment->gradient);
   }
+  CS_ASSERT_TRUE(!max_grad_norm_.has_value() || order.size() <= 1,
+                 "gradient clipping needs one dtype and one set of hyper-parameters for all parameters");
   for (const auto &key : order) {
     const auto &group = groups.at(key);
-    optimizer::AdamW::step(scheduler, group.states, group.parameters, group.gradients);
+    last_grad_norm_ = optimizer::AdamW::step(scheduler, group.states, group.parameters, group.gradients,
+                                             max_grad_norm_, 2.0);
   }
 }
 }  // namespace cs::module

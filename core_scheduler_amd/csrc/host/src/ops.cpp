@@ -21,6 +21,7 @@
 #include "compute/embedding.h"
 #include "compute/gelu.h"
 #include "compute/layer_norm.h"
+#include "compute/utils.h"
 #include "cs_hip_kernels.h"
 #include "logger.h"
 #include "memory/to_torch.h"
@@ -504,6 +505,73 @@ Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<Sta
 }
 }  // namespace compute
 
+namespace {
+// Lays the descriptor table out in pinned host memory and copies it to the device on the
+// current stream; libtorch keeps the pinned block alive until the copy has run.
+at::Tensor upload_table(const std::vector<cs_adamw_tensor> &descs, const int dtype, const at::TensorOptions &like,
+                        int64_t *slots, const char *who) {
+  const size_t bytes = cs_adamw_multi_table_bytes(static_cast<int64_t>(descs.size()));
+  at::Tensor host = at::empty({static_cast<int64_t>(bytes)}, at::TensorOptions().dtype(at::kByte).pinned_memory(true));
+  check(cs_adamw_multi_build_table(descs.data(), static_cast<int64_t>(descs.size()), dtype, host.data_ptr(), bytes,
+                                   slots),
+        who);
+  at::Tensor table = at::empty({static_cast<int64_t>(bytes)}, like.dtype(at::kByte));
+  table.copy_(host, /*non_blocking=*/true);
+  return table;
+}
+}  // namespace
+
+// =================================================================== Utils
+namespace compute::Utils {
+Tensor clip_grad_norm_(const Scheduler &scheduler, const std::vector<Tensor> &tensor, const double max_norm,
+                       const double norm_type) {
+  struct Body final : Task::Impl {
+    double max_norm, norm_type;
+    Body(std::vector<Tensor> out /* gradients..., total_norm */, std::vector<ReadOnlyTensor> in /* gradients */,
+         const double max_norm, const double norm_type)
+        : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, max_norm{max_norm}, norm_type{norm_type} {}
+    void operator()() const override {
+      // the gradient table of the optimizer step, with the gradient standing in for the other pointers
+      std::vector<cs_adamw_tensor> descs;
+      int dtype = -1;
+      at::TensorOptions like;
+      for (const auto &in : input()) {
+        const at::Tensor &g = T(in);
+        if (!g.defined()) continue;
+        TORCH_CHECK(g.is_contiguous(), "clip_grad_norm_ needs contiguous gradients");
+        const int dt = dtype_of(g.scalar_type());
+        CS_ASSERT_TRUE(dtype < 0 || dt == dtype, "clip_grad_norm_ needs one dtype");
+        dtype = dt;
+        like = g.options();
+        descs.push_back({g.data_ptr(), g.data_ptr(), g.data_ptr(), g.data_ptr(), nullptr, g.numel()});
+      }
+      if (descs.empty()) return;
+      int64_t slots = 0;
+      at::Tensor table = upload_table(descs, dtype, like, &slots, name());
+      const auto count = static_cast<int64_t>(descs.size());
+      at::Tensor norm = at::empty({}, like.dtype(at::kFloat)), coef = at::empty({}, like.dtype(at::kFloat));
+      const size_t ws_bytes = cs_grad_norm_multi_workspace_bytes(slots);
+      at::Tensor ws = at::empty({static_cast<int64_t>(ws_bytes)}, like.dtype(at::kByte));
+      check(cs_grad_norm_multi(table.data_ptr(), count, slots, dtype, norm_type, max_norm, ws.data_ptr(), ws_bytes,
+                               norm.data_ptr<float>(), coef.data_ptr<float>(), current_stream()),
+            name());
+      check(cs_grad_scale_multi(table.data_ptr(), count, slots, dtype, coef.data_ptr<float>(), current_stream()), name());
+      T(output().back()) = norm;
+      intermediate().push_back(table);
+      intermediate().push_back(ws);
+      intermediate().push_back(coef);
+    }
+    [[nodiscard]] const char *name() const override { return "cs::compute::Utils::clip_grad_norm_"; }
+  };
+  Tensor total_norm;
+  std::vector<Tensor> outs{tensor};
+  outs.push_back(total_norm);
+  scheduler.impl()->submit(Task{std::make_shared<Body>(
+      std::move(outs), std::vector<ReadOnlyTensor>{tensor.begin(), tensor.end()}, max_norm, norm_type)});
+  return total_norm;
+}
+}  // namespace compute::Utils
+
 // =================================================================== AdamW
 namespace optimizer {
 AdamW::State::State(const Tensors &tensors, const Options &options) : tensors{tensors}, options{options} {}
@@ -565,14 +633,27 @@ void AdamW::step(const Scheduler &scheduler, const std::shared_ptr<module::Optim
 
 void AdamW::step(const Scheduler &scheduler, const std::vector<std::shared_ptr<module::OptimizerState>> &states,
                  const std::vector<Tensor> &ws, const std::vector<ReadOnlyTensor> &dws) {
+  (void)step(scheduler, states, ws, dws, c10::nullopt, 2.0);
+}
+
+Tensor AdamW::step(const Scheduler &scheduler, const std::vector<std::shared_ptr<module::OptimizerState>> &states,
+                   const std::vector<Tensor> &ws, const std::vector<ReadOnlyTensor> &dws,
+                   const c10::optional<double> max_grad_norm, const double norm_type) {
   CS_ASSERT_TRUE(states.size() == ws.size() && ws.size() == dws.size(), "one state and one gradient per parameter");
-  if (states.empty()) return;
+  Tensor total_norm;
+  if (states.empty()) return total_norm;
   struct Body final : Task::Impl {
     State::Options options;
     size_t n;
-    Body(std::vector<Tensor> out /* n x (w, m, v, v_max) */, std::vector<ReadOnlyTensor> in /* n x dw */,
-         const State::Options &o, const size_t count)
-        : Task::Impl{std::move(out), std::move(in), kAssist, kCompute}, options{o}, n{count} {}
+    c10::optional<double> max_norm;
+    double norm_type;
+    Body(std::vector<Tensor> out /* n x (w, m, v, v_max), total_norm */, std::vector<ReadOnlyTensor> in /* n x dw */,
+         const State::Options &o, const size_t count, const c10::optional<double> max_norm, const double norm_type)
+        : Task::Impl{std::move(out), std::move(in), kAssist, kCompute},
+          options{o},
+          n{count},
+          max_norm{max_norm},
+          norm_type{norm_type} {}
     void operator()() const override {
       std::vector<cs_adamw_tensor> descs;
       descs.reserve(n);
@@ -595,18 +676,30 @@ void AdamW::step(const Scheduler &scheduler, const std::vector<std::shared_ptr<m
                          options.amsgrad ? T(output()[4 * i + 3]).data_ptr() : nullptr, g.numel()});
       }
       if (descs.empty()) return;
-      const size_t bytes = cs_adamw_multi_table_bytes(static_cast<int64_t>(descs.size()));
-      at::Tensor host = at::empty({static_cast<int64_t>(bytes)}, at::TensorOptions().dtype(at::kByte).pinned_memory(true));
       int64_t slots = 0;
-      check(cs_adamw_multi_build_table(descs.data(), static_cast<int64_t>(descs.size()), dtype, host.data_ptr(), bytes,
-                                       &slots),
-            name());
-      at::Tensor table = at::empty({static_cast<int64_t>(bytes)}, like.dtype(at::kByte));
-      table.copy_(host, /*non_blocking=*/true);  // a copy on the current stream; libtorch keeps `host` alive
-      check(cs_adamw_multi_step(table.data_ptr(), static_cast<int64_t>(descs.size()), slots, dtype,
-                                options.amsgrad ? 1 : 0, options.lr, options.beta1, options.beta2, options.eps,
-                                options.weight_decay, options.t, current_stream()),
-            name());
+      at::Tensor table = upload_table(descs, dtype, like, &slots, name());
+      const auto count = static_cast<int64_t>(descs.size());
+      if (max_norm.has_value()) {
+        // global norm first (two small launches), then the step scales each gradient as it reads it
+        at::Tensor norm = at::empty({}, like.dtype(at::kFloat)), coef = at::empty({}, like.dtype(at::kFloat));
+        const size_t ws_bytes = cs_grad_norm_multi_workspace_bytes(slots);
+        at::Tensor ws = at::empty({static_cast<int64_t>(ws_bytes)}, like.dtype(at::kByte));
+        check(cs_grad_norm_multi(table.data_ptr(), count, slots, dtype, norm_type, *max_norm, ws.data_ptr(), ws_bytes,
+                                 norm.data_ptr<float>(), coef.data_ptr<float>(), current_stream()),
+              name());
+        check(cs_adamw_multi_step_clipped(table.data_ptr(), count, slots, dtype, options.amsgrad ? 1 : 0, options.lr,
+                                          options.beta1, options.beta2, options.eps, options.weight_decay, options.t,
+                                          coef.data_ptr<float>(), current_stream()),
+              name());
+        T(output().back()) = norm;
+        intermediate().push_back(ws);
+        intermediate().push_back(coef);
+      } else {
+        check(cs_adamw_multi_step(table.data_ptr(), count, slots, dtype, options.amsgrad ? 1 : 0, options.lr,
+                                  options.beta1, options.beta2, options.eps, options.weight_decay, options.t,
+                                  current_stream()),
+              name());
+      }
       intermediate().push_back(table);
     }
     [[nodiscard]] const char *name() const override { return "cs::optimizer::AdamW::step(all)"; }
@@ -632,7 +725,10 @@ void AdamW::step(const Scheduler &scheduler, const std::vector<std::shared_ptr<m
     outs.push_back(s->tensors.v_max);
     ins.push_back(dws[i]);
   }
-  scheduler.impl()->submit(Task{std::make_shared<Body>(std::move(outs), std::move(ins), *first, states.size())});
+  outs.push_back(total_norm);
+  scheduler.impl()->submit(
+      Task{std::make_shared<Body>(std::move(outs), std::move(ins), *first, states.size(), max_grad_norm, norm_type)});
+  return total_norm;
 }
 }  // namespace optimizer
 

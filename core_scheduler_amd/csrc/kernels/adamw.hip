@@ -15,6 +15,8 @@
 
 #include <math.h>
 
+#include <cmath>
+
 namespace cs_hip {
 namespace {
 
@@ -35,12 +37,16 @@ __device__ __forceinline__ double dev_sqrt<double>(double x) {
 }
 
 // One element, reference operation order.
+// `gscale` is the gradient-clipping coefficient (1 when not clipping).  The scaled gradient
+// is rounded to the storage type first, as the reference's in-place clip leaves it
+// (src/compute/utils.cpp:733-736); multiplying by 1 changes nothing.
 template <typename T, bool AMSGRAD>
 __device__ __forceinline__ void adam_update(T &w, T &m, T &v, T &vmax, const T g_in,
-                                            const AdamHyper<typename Acc<T>::type> &h) {
+                                            const AdamHyper<typename Acc<T>::type> &h,
+                                            const typename Acc<T>::type gscale) {
   using U = typename Acc<T>::type;
   const U one = (U)1;
-  const U g = to_acc(g_in);
+  const U g = to_acc(from_acc<T>(to_acc(g_in) * gscale));
   const U w0 = to_acc(w);
   const U theta = w0 - h.lr * h.wd * w0;
   const U m_t = h.beta1 * to_acc(m) + (one - h.beta1) * g;
@@ -74,7 +80,8 @@ __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restric
                                            T *__restrict__ m, T *__restrict__ v,
                                            T *__restrict__ vmax, int64_t begin, int64_t end,
                                            bool vec_ok,
-                                           const AdamHyper<typename Acc<T>::type> &h) {
+                                           const AdamHyper<typename Acc<T>::type> &h,
+                                           const typename Acc<T>::type gscale) {
   constexpr int VN = Vec16<T>::n;
   const int tid = threadIdx.x;
   if (vec_ok && end - begin == adam_chunk_elems<T>()) {
@@ -94,7 +101,7 @@ __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restric
       const int64_t off = begin + ((int64_t)u * kAdamThreads + tid) * VN;
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
-        adam_update<T, AMSGRAD>(vw[u].e[k], vm[u].e[k], vv[u].e[k], vx[u].e[k], vg[u].e[k], h);
+        adam_update<T, AMSGRAD>(vw[u].e[k], vm[u].e[k], vv[u].e[k], vx[u].e[k], vg[u].e[k], h, gscale);
       }
       store16_stream(w + off, vw[u]);
       store16_stream(m + off, vm[u]);
@@ -107,7 +114,7 @@ __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restric
   for (int64_t i = begin + tid; i < end; i += kAdamThreads) {
     T wi = w[i], mi = m[i], vi = v[i], xi{};
     if constexpr (AMSGRAD) xi = vmax[i];
-    adam_update<T, AMSGRAD>(wi, mi, vi, xi, dw[i], h);
+    adam_update<T, AMSGRAD>(wi, mi, vi, xi, dw[i], h, gscale);
     w[i] = wi;
     m[i] = mi;
     v[i] = vi;
@@ -122,7 +129,7 @@ __global__ __launch_bounds__(kAdamThreads) void adamw_flat_kernel(
   const int64_t chunk = adam_chunk_elems<T>();
   const int64_t begin = (int64_t)blockIdx.x * chunk;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
-  adam_chunk<T, AMSGRAD>(w, dw, m, v, vmax, begin, end, vec_ok, h);
+  adam_chunk<T, AMSGRAD>(w, dw, m, v, vmax, begin, end, vec_ok, h, (typename Acc<T>::type)1);
 }
 
 // ---------------------------------------------------------- multi-tensor
@@ -146,12 +153,10 @@ __host__ __device__ inline int64_t slot_array_len(int64_t n_tensors) {
   return (n_tensors + 1 + 7) / 8 * 8;
 }
 
-template <typename T, bool AMSGRAD>
-__global__ __launch_bounds__(kAdamThreads) void adamw_multi_kernel(
-    const int64_t *__restrict__ table, int n_tensors, AdamHyper<typename Acc<T>::type> h) {
-  const int64_t slot = blockIdx.x;
-  // binary search over the prefix array; wave-uniform, so it runs on the
-  // scalar unit out of the constant cache
+// The tensor that owns workgroup slot `slot`: binary search over the prefix array;
+// wave-uniform, so it runs on the scalar unit out of the constant cache.
+__device__ __forceinline__ int tensor_of_slot(const int64_t *__restrict__ table, int n_tensors,
+                                              int64_t slot) {
   int lo = 0, hi = n_tensors;  // invariant: first_slot[lo] <= slot < first_slot[hi]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -161,15 +166,147 @@ __global__ __launch_bounds__(kAdamThreads) void adamw_multi_kernel(
       hi = mid;
     }
   }
+  return lo;
+}
+
+// `clip` points at the clipping coefficient in device memory (written by the norm launches
+// that precede this one on the stream), or is null.
+template <typename T, bool AMSGRAD>
+__global__ __launch_bounds__(kAdamThreads) void adamw_multi_kernel(
+    const int64_t *__restrict__ table, int n_tensors, AdamHyper<typename Acc<T>::type> h,
+    const float *__restrict__ clip) {
+  using U = typename Acc<T>::type;
+  const int64_t slot = blockIdx.x;
+  const int lo = tensor_of_slot(table, n_tensors, slot);
   const DevTensor *desc =
       reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
   const int64_t chunk = adam_chunk_elems<T>();
   const int64_t begin = (slot - table[lo]) * chunk;
   const int64_t n = desc->n;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
+  const U gscale = clip ? (U)*clip : (U)1;
   adam_chunk<T, AMSGRAD>(static_cast<T *>(desc->w), static_cast<const T *>(desc->dw),
                          static_cast<T *>(desc->m), static_cast<T *>(desc->v),
-                         static_cast<T *>(desc->vmax), begin, end, desc->vec_ok != 0, h);
+                         static_cast<T *>(desc->vmax), begin, end, desc->vec_ok != 0, h, gscale);
+}
+
+// ------------------------------------------------- global gradient norm
+// Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746): total = ||all gradients||_p,
+// coefficient = min(1, max_norm / (total + 1e-6)), gradients *= coefficient.
+// Pass 1 walks the same table as the step: each workgroup reduces its chunk of one
+// gradient to a partial (sum of squares, or largest magnitude for the infinity norm).
+// Pass 2 adds the partials in slot order in double, so the result does not depend on
+// scheduling, and writes the norm and the coefficient.
+template <typename T, bool INF>
+__global__ __launch_bounds__(kAdamThreads) void grad_norm_partial_kernel(
+    const int64_t *__restrict__ table, int n_tensors, float *__restrict__ partial) {
+  constexpr int VN = Vec16<T>::n;
+  const int64_t slot = blockIdx.x;
+  const int lo = tensor_of_slot(table, n_tensors, slot);
+  const DevTensor *desc =
+      reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
+  const T *g = static_cast<const T *>(desc->dw);
+  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t begin = (slot - table[lo]) * chunk;
+  const int64_t n = desc->n;
+  const int64_t end = begin + chunk < n ? begin + chunk : n;
+  const int tid = threadIdx.x;
+  float acc = 0.f;
+  auto take = [&](const T x) {
+    const float f = (float)to_acc(x);
+    if constexpr (INF) {
+      acc = fmaxf(acc, fabsf(f));
+    } else {
+      acc += f * f;
+    }
+  };
+  if (is_aligned16(g) && end - begin == chunk) {
+    Vec16<T> v[kAdamUnroll];
+#pragma unroll
+    for (int u = 0; u < kAdamUnroll; ++u)
+      v[u] = load16(g + begin + ((int64_t)u * kAdamThreads + tid) * VN);  // read again by the step: keep it cached
+#pragma unroll
+    for (int u = 0; u < kAdamUnroll; ++u)
+#pragma unroll
+      for (int k = 0; k < VN; ++k) take(v[u].e[k]);
+  } else {
+    for (int64_t i = begin + tid; i < end; i += kAdamThreads) take(g[i]);
+  }
+  __shared__ float scratch[kAdamThreads / kWave];
+  float total;
+  if constexpr (INF) {
+    total = block_reduce(acc, MaxOp{}, 0.f, scratch);
+  } else {
+    total = block_reduce(acc, SumOp{}, 0.f, scratch);
+  }
+  if (tid == 0) partial[slot] = total;
+}
+
+template <bool INF>
+__global__ __launch_bounds__(1024) void grad_norm_final_kernel(const float *__restrict__ partial,
+                                                               int64_t n_slots, float max_norm,
+                                                               float *__restrict__ total_norm,
+                                                               float *__restrict__ clip) {
+  __shared__ double scratch[1024 / kWave];
+  const int tid = threadIdx.x;
+  // thread t owns the contiguous run of slots [t*per, (t+1)*per): a fixed order
+  const int64_t per = (n_slots + 1023) / 1024;
+  const int64_t lo = (int64_t)tid * per;
+  const int64_t hi = lo + per < n_slots ? lo + per : n_slots;
+  double acc = 0.;
+  for (int64_t i = lo; i < hi; ++i) {
+    const double p = (double)partial[i];
+    if constexpr (INF) {
+      acc = p > acc ? p : acc;
+    } else {
+      acc += p;
+    }
+  }
+  double total;
+  if constexpr (INF) {
+    total = block_reduce(acc, MaxOp{}, 0., scratch);
+  } else {
+    total = block_reduce(acc, SumOp{}, 0., scratch);
+  }
+  if (tid == 0) {
+    const float norm = INF ? (float)total : (float)sqrt(total);
+    *total_norm = norm;
+    // in float, as the reference's tensor ops are: max_norm / (norm + 1e-6), clamped to 1
+    const float coef = max_norm / (norm + 1e-6f);
+    *clip = coef < 1.0f ? coef : 1.0f;
+  }
+}
+
+// gradients *= coefficient, in place (what the reference's clip leaves behind)
+template <typename T>
+__global__ __launch_bounds__(kAdamThreads) void grad_scale_kernel(const int64_t *__restrict__ table,
+                                                                  int n_tensors,
+                                                                  const float *__restrict__ clip) {
+  using U = typename Acc<T>::type;
+  constexpr int VN = Vec16<T>::n;
+  const int64_t slot = blockIdx.x;
+  const int lo = tensor_of_slot(table, n_tensors, slot);
+  const DevTensor *desc =
+      reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
+  T *g = static_cast<T *>(const_cast<void *>(desc->dw));
+  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t begin = (slot - table[lo]) * chunk;
+  const int64_t n = desc->n;
+  const int64_t end = begin + chunk < n ? begin + chunk : n;
+  const int tid = threadIdx.x;
+  const U scale = (U)*clip;
+  if (is_aligned16(g) && end - begin == chunk) {
+#pragma unroll
+    for (int u = 0; u < kAdamUnroll; ++u) {
+      T *p = g + begin + ((int64_t)u * kAdamThreads + tid) * VN;
+      Vec16<T> v = load16(p);
+#pragma unroll
+      for (int k = 0; k < VN; ++k) v.e[k] = from_acc<T>(to_acc(v.e[k]) * scale);
+      store16(p, v);
+    }
+  } else {
+    for (int64_t i = begin + tid; i < end; i += kAdamThreads) g[i] = from_acc<T>(to_acc(g[i]) * scale);
+  }
 }
 
 template <typename U>
@@ -222,16 +359,17 @@ int launch_flat(void *w, const void *dw, void *m, void *v, void *vmax, int64_t n
 
 template <typename T>
 int launch_multi(const void *table, int64_t n_tensors, int64_t n_slots, int amsgrad, double lr,
-                 double beta1, double beta2, double eps, double wd, int64_t t, hipStream_t s) {
+                 double beta1, double beta2, double eps, double wd, int64_t t, const float *clip,
+                 hipStream_t s) {
   using U = typename Acc<T>::type;
   const AdamHyper<U> h = make_hyper<U>(lr, beta1, beta2, eps, wd, t);
   const int64_t *tab = static_cast<const int64_t *>(table);
   if (amsgrad) {
     adamw_multi_kernel<T, true>
-        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h);
+        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h, clip);
   } else {
     adamw_multi_kernel<T, false>
-        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h);
+        <<<dim3((unsigned)n_slots), dim3(kAdamThreads), 0, s>>>(tab, (int)n_tensors, h, clip);
   }
   return launch_status();
 }
@@ -311,9 +449,10 @@ extern "C" int cs_adamw_multi_build_table(const cs_adamw_tensor *tensors, int64_
   return CS_OK;
 }
 
-extern "C" int cs_adamw_multi_step(const void *device_table, int64_t n_tensors, int64_t n_slots,
-                                   int dtype, int amsgrad, double lr, double beta1, double beta2,
-                                   double eps, double weight_decay, int64_t t, void *stream) {
+namespace {
+int multi_step(const void *device_table, int64_t n_tensors, int64_t n_slots, int dtype, int amsgrad,
+               double lr, double beta1, double beta2, double eps, double weight_decay, int64_t t,
+               const float *clip, void *stream) {
   if (n_tensors < 0 || n_slots < 0) return CS_ERR_INVALID_ARGUMENT;
   if (n_tensors == 0 || n_slots == 0) return CS_OK;
   if (!device_table || !aligned_to(device_table, 16)) return CS_ERR_INVALID_ARGUMENT;
@@ -322,16 +461,103 @@ extern "C" int cs_adamw_multi_step(const void *device_table, int64_t n_tensors, 
   switch (dtype) {
     case CS_F32:
       return launch_multi<float>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
-                                 weight_decay, t, s);
+                                 weight_decay, t, clip, s);
     case CS_F64:
       return launch_multi<double>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
-                                  weight_decay, t, s);
+                                  weight_decay, t, clip, s);
     case CS_F16:
       return launch_multi<f16_t>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
-                                 weight_decay, t, s);
+                                 weight_decay, t, clip, s);
     case CS_BF16:
       return launch_multi<bf16_t>(device_table, n_tensors, n_slots, amsgrad, lr, beta1, beta2, eps,
-                                  weight_decay, t, s);
+                                  weight_decay, t, clip, s);
   }
   return CS_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+int launch_norm(const void *table, int64_t n_tensors, int64_t n_slots, bool inf, float max_norm,
+                float *partial, float *total_norm, float *clip, hipStream_t s) {
+  const int64_t *tab = static_cast<const int64_t *>(table);
+  const dim3 grid((unsigned)n_slots), block(kAdamThreads);
+  if (inf) {
+    grad_norm_partial_kernel<T, true><<<grid, block, 0, s>>>(tab, (int)n_tensors, partial);
+    grad_norm_final_kernel<true><<<dim3(1), dim3(1024), 0, s>>>(partial, n_slots, max_norm, total_norm, clip);
+  } else {
+    grad_norm_partial_kernel<T, false><<<grid, block, 0, s>>>(tab, (int)n_tensors, partial);
+    grad_norm_final_kernel<false><<<dim3(1), dim3(1024), 0, s>>>(partial, n_slots, max_norm, total_norm, clip);
+  }
+  return launch_status();
+}
+}  // namespace
+
+extern "C" int cs_adamw_multi_step(const void *device_table, int64_t n_tensors, int64_t n_slots,
+                                   int dtype, int amsgrad, double lr, double beta1, double beta2,
+                                   double eps, double weight_decay, int64_t t, void *stream) {
+  return multi_step(device_table, n_tensors, n_slots, dtype, amsgrad, lr, beta1, beta2, eps,
+                    weight_decay, t, nullptr, stream);
+}
+
+extern "C" int cs_adamw_multi_step_clipped(const void *device_table, int64_t n_tensors,
+                                           int64_t n_slots, int dtype, int amsgrad, double lr,
+                                           double beta1, double beta2, double eps,
+                                           double weight_decay, int64_t t, const float *clip_coef,
+                                           void *stream) {
+  if (!clip_coef || !aligned_to(clip_coef, 4)) return CS_ERR_INVALID_ARGUMENT;
+  return multi_step(device_table, n_tensors, n_slots, dtype, amsgrad, lr, beta1, beta2, eps,
+                    weight_decay, t, clip_coef, stream);
+}
+
+extern "C" size_t cs_grad_norm_multi_workspace_bytes(int64_t n_slots) {
+  if (n_slots <= 0) return 0;
+  return ((size_t)n_slots * sizeof(float) + 255) / 256 * 256;
+}
+
+extern "C" int cs_grad_norm_multi(const void *device_table, int64_t n_tensors, int64_t n_slots,
+                                  int dtype, double norm_type, double max_norm, void *workspace,
+                                  size_t workspace_bytes, float *total_norm, float *clip_coef,
+                                  void *stream) {
+  if (n_tensors <= 0 || n_slots <= 0) return CS_ERR_INVALID_ARGUMENT;
+  const bool inf = std::isinf(norm_type) && norm_type > 0;
+  if (!inf && norm_type != 2.0) return CS_ERR_UNSUPPORTED;
+  if (!device_table || !aligned_to(device_table, 16) || !total_norm || !clip_coef ||
+      !aligned_to(total_norm, 4) || !aligned_to(clip_coef, 4))
+    return CS_ERR_INVALID_ARGUMENT;
+  if (n_slots > 0x7fffffffLL || n_tensors > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  if (!workspace || workspace_bytes < cs_grad_norm_multi_workspace_bytes(n_slots) ||
+      !aligned_to(workspace, 16))
+    return CS_ERR_WORKSPACE;
+  hipStream_t s = as_stream(stream);
+  float *partial = static_cast<float *>(workspace);
+  const float mx = (float)max_norm;
+  switch (dtype) {
+    case CS_F32:
+      return launch_norm<float>(device_table, n_tensors, n_slots, inf, mx, partial, total_norm, clip_coef, s);
+    case CS_F64:
+      return launch_norm<double>(device_table, n_tensors, n_slots, inf, mx, partial, total_norm, clip_coef, s);
+    case CS_F16:
+      return launch_norm<f16_t>(device_table, n_tensors, n_slots, inf, mx, partial, total_norm, clip_coef, s);
+    case CS_BF16:
+      return launch_norm<bf16_t>(device_table, n_tensors, n_slots, inf, mx, partial, total_norm, clip_coef, s);
+  }
+  return CS_ERR_UNSUPPORTED;
+}
+
+extern "C" int cs_grad_scale_multi(const void *device_table, int64_t n_tensors, int64_t n_slots,
+                                   int dtype, const float *clip_coef, void *stream) {
+  if (n_tensors <= 0 || n_slots <= 0) return CS_ERR_INVALID_ARGUMENT;
+  if (!device_table || !aligned_to(device_table, 16) || !clip_coef || !aligned_to(clip_coef, 4))
+    return CS_ERR_INVALID_ARGUMENT;
+  if (n_slots > 0x7fffffffLL || n_tensors > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  hipStream_t s = as_stream(stream);
+  const int64_t *tab = static_cast<const int64_t *>(device_table);
+  const dim3 grid((unsigned)n_slots), block(kAdamThreads);
+  switch (dtype) {
+    case CS_F32: grad_scale_kernel<float><<<grid, block, 0, s>>>(tab, (int)n_tensors, clip_coef); break;
+    case CS_F64: grad_scale_kernel<double><<<grid, block, 0, s>>>(tab, (int)n_tensors, clip_coef); break;
+    case CS_F16: grad_scale_kernel<f16_t><<<grid, block, 0, s>>>(tab, (int)n_tensors, clip_coef); break;
+    case CS_BF16: grad_scale_kernel<bf16_t><<<grid, block, 0, s>>>(tab, (int)n_tensors, clip_coef); break;
+    default: return CS_ERR_UNSUPPORTED;
+  }
+  return launch_status();
 }

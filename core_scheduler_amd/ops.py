@@ -115,15 +115,50 @@ class MultiTensorAdamW:
         self._grads = grads  # keep them alive: the table holds their addresses
         self._table.copy_(self._host, non_blocking=True)
 
-    def step(self):
+    def step(self, max_grad_norm=None, norm_type=2.0):
+        """One launch for every parameter.  With `max_grad_norm`, the global gradient norm is
+        taken first (two small launches) and the step applies the clipping coefficient to the
+        gradients as it reads them; returns the norm as a 0-d device tensor then."""
         self.t += 1
         lib = _capi.load()
+        n = len(self.params)
         with torch.cuda.device(self.dev):
-            code = lib.cs_adamw_multi_step(_ptr(self._table), len(self.params), self._slots,
-                                           _DTYPES[self.dtype], int(self.amsgrad), self.lr, self.beta1,
-                                           self.beta2, self.eps, self.weight_decay, self.t,
-                                           _stream(self.dev))
-        _capi.check("cs_adamw_multi_step", code)
+            if max_grad_norm is None:
+                code = lib.cs_adamw_multi_step(_ptr(self._table), n, self._slots, _DTYPES[self.dtype],
+                                               int(self.amsgrad), self.lr, self.beta1, self.beta2, self.eps,
+                                               self.weight_decay, self.t, _stream(self.dev))
+                _capi.check("cs_adamw_multi_step", code)
+                return None
+            norm = self.grad_norm(max_grad_norm, norm_type)
+            code = lib.cs_adamw_multi_step_clipped(_ptr(self._table), n, self._slots, _DTYPES[self.dtype],
+                                                   int(self.amsgrad), self.lr, self.beta1, self.beta2, self.eps,
+                                                   self.weight_decay, self.t, _ptr(self._clip), _stream(self.dev))
+            _capi.check("cs_adamw_multi_step_clipped", code)
+            return norm
+
+    def grad_norm(self, max_norm, norm_type=2.0):
+        """Global norm of all gradients; leaves the clipping coefficient in `self._clip`."""
+        lib = _capi.load()
+        nbytes = lib.cs_grad_norm_multi_workspace_bytes(self._slots)
+        if getattr(self, "_norm_ws", None) is None or self._norm_ws.numel() < nbytes:
+            self._norm_ws = torch.empty(nbytes, dtype=torch.uint8, device=self.dev)
+            self._clip = torch.empty((), dtype=torch.float32, device=self.dev)
+        norm = torch.empty((), dtype=torch.float32, device=self.dev)
+        with torch.cuda.device(self.dev):
+            code = lib.cs_grad_norm_multi(_ptr(self._table), len(self.params), self._slots, _DTYPES[self.dtype],
+                                          float(norm_type), float(max_norm), _ptr(self._norm_ws), nbytes,
+                                          _ptr(norm), _ptr(self._clip), _stream(self.dev))
+        _capi.check("cs_grad_norm_multi", code)
+        return norm
+
+    def clip_grad_norm_(self, max_norm, norm_type=2.0):
+        """The reference's Utils::clip_grad_norm_: scales the gradients in place, returns the norm."""
+        norm = self.grad_norm(max_norm, norm_type)
+        with torch.cuda.device(self.dev):
+            code = _capi.load().cs_grad_scale_multi(_ptr(self._table), len(self.params), self._slots,
+                                                    _DTYPES[self.dtype], _ptr(self._clip), _stream(self.dev))
+        _capi.check("cs_grad_scale_multi", code)
+        return norm
 
 
 # ------------------------------------------------------------------- GeLU

@@ -124,6 +124,33 @@ int cs_adamw_multi_step(const void *device_table, int64_t n_tensors,
                         double beta1, double beta2, double eps,
                         double weight_decay, int64_t t, void *stream);
 
+/* Global gradient-norm clipping over the same table — Utils::clip_grad_norm_
+ * (src/compute/utils.cpp:700-746), which the GPT-2 example leaves as a TODO
+ * (example/gpt2/gpt2_single_device.cpp:706).  cs_grad_norm_multi writes
+ *   *total_norm = || all gradients ||_p   (p = 2, or +infinity)
+ *   *clip_coef  = min(1, max_norm / (total_norm + 1e-6))      (float arithmetic)
+ * to device memory with two launches: one partial per workgroup slot, then a
+ * sum in slot order in double (the result does not depend on scheduling).
+ * The reference then multiplies every gradient in place; that pass is
+ * cs_grad_scale_multi.  cs_adamw_multi_step_clipped instead reads the
+ * coefficient inside the step and applies it to each gradient as it is
+ * loaded (rounded to the gradient's type first, so the update is the one the
+ * in-place clip followed by the plain step gives), leaving the gradients as
+ * they were: one 4 B/parameter read instead of a read and a write more. */
+size_t cs_grad_norm_multi_workspace_bytes(int64_t n_slots);
+int cs_grad_norm_multi(const void *device_table, int64_t n_tensors,
+                       int64_t n_slots, int dtype, double norm_type,
+                       double max_norm, void *workspace, size_t workspace_bytes,
+                       float *total_norm, float *clip_coef, void *stream);
+int cs_grad_scale_multi(const void *device_table, int64_t n_tensors,
+                        int64_t n_slots, int dtype, const float *clip_coef,
+                        void *stream);
+int cs_adamw_multi_step_clipped(const void *device_table, int64_t n_tensors,
+                                int64_t n_slots, int dtype, int amsgrad,
+                                double lr, double beta1, double beta2,
+                                double eps, double weight_decay, int64_t t,
+                                const float *clip_coef, void *stream);
+
 /* ------------------------------------------------------------------------
  * GeLU
  * replaces at::gelu / at::gelu_backward in the task bodies of

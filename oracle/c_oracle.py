@@ -65,6 +65,22 @@ def adamw_step(w, dw, m, v, *, lr, beta1, beta2, eps, weight_decay, t, v_max=Non
     return ww.to(dt), mw.to(dt), vw.to(dt), (xw.to(dt) if xw is not None else None)
 
 
+def clip_grad_norm(grads, max_norm, norm_type=2.0):
+    """(scaled gradients in their dtype, total_norm, clip_coef); the inputs are not modified.
+    16-bit gradients are widened, scaled in float and rounded once, as an in-place multiply does."""
+    wide = [_wide(g) for g in grads]
+    sfx = wide[0][1]
+    bufs = [w for w, _ in wide]
+    n = len(bufs)
+    ptrs = (ctypes.c_void_p * n)(*[b.data_ptr() for b in bufs])
+    sizes = (ctypes.c_int64 * n)(*[b.numel() for b in bufs])
+    real = ctypes.c_double if sfx == "f64" else ctypes.c_float
+    total, coef = real(0), real(0)
+    _call("oracle_clip_grad_norm", sfx, ptrs, sizes, I64(n), INT(1 if norm_type == float("inf") else 0),
+          DBL(max_norm), INT(1), ctypes.byref(total), ctypes.byref(coef))
+    return [b.to(g.dtype).reshape(g.shape) for b, g in zip(bufs, grads)], total.value, coef.value
+
+
 def gelu_forward(x, approximate="none"):
     xw, sfx = _wide(x)
     y = torch.empty_like(xw)

@@ -43,6 +43,36 @@ void FN(oracle_adamw_step)(REAL *w, const REAL *dw, REAL *m, REAL *v, REAL *v_ma
   }
 }
 
+/* ---- gradient clipping: src/compute/utils.cpp:700-746 (Utils::clip_grad_norm_)
+ * total = || hstack(all gradients) ||_p for p = 2 (inf_norm == 0) or +infinity
+ * (inf_norm != 0); coefficient = min(1, max_norm / (total + 1e-6)) in the tensors'
+ * arithmetic type; every gradient is multiplied by it in place when `scale` is set.
+ * The sum of squares is accumulated in double and narrowed once (see the header). */
+void FN(oracle_clip_grad_norm)(REAL *const *grads, const int64_t *sizes, int64_t n_tensors,
+                               int inf_norm, double max_norm_d, int scale, REAL *total_norm,
+                               REAL *clip_coef) {
+  double acc = 0.;
+  for (int64_t t = 0; t < n_tensors; ++t) {
+    for (int64_t i = 0; i < sizes[t]; ++i) {
+      const double g = (double)grads[t][i];
+      if (inf_norm) {
+        acc = fabs(g) > acc ? fabs(g) : acc;
+      } else {
+        acc += g * g;
+      }
+    }
+  }
+  const REAL total = (REAL)(inf_norm ? acc : sqrt(acc));
+  REAL coef = (REAL)max_norm_d / (total + (REAL)1e-6);
+  if (coef > (REAL)1) coef = (REAL)1;
+  *total_norm = total;
+  *clip_coef = coef;
+  if (scale) {
+    for (int64_t t = 0; t < n_tensors; ++t)
+      for (int64_t i = 0; i < sizes[t]; ++i) grads[t][i] = grads[t][i] * coef;
+  }
+}
+
 /* ---- GeLU: src/compute/gelu.cpp:39 (at::gelu), :61-62 (at::gelu_backward)
  * mode 0 = exact: x * 0.5 * (1 + erf(x / sqrt 2)); derivative cdf + x * pdf.
  * mode 1 = at::gelu(x, "tanh"): 0.5 x (1 + tanh(kBeta (x + kKappa x^3))),

@@ -152,6 +152,61 @@ def test_adamw_gpt2_small_ten_steps(ops, co):
     assert_close(torch.cat([x.flatten() for x in opt.v]), v, atol=1e-13, name="v")
 
 
+@pytest.mark.parametrize("norm_type", [2.0, float("inf")])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_clip_grad_norm_and_clipped_step(ops, co, norm_type, dtype):
+    """Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746): norm, coefficient, in-place scaling,
+    and the step that applies the coefficient while it reads the gradients."""
+    shapes = [(7,), (4096,), (33, 129), (4097,), (1,), (3, 5, 7), (50000,)]
+    ws = [randn(s, 20 + i, std=0.02, dtype=dtype) for i, s in enumerate(shapes)]
+    gs = [randn(s, 40 + i, std=1e-1, dtype=dtype) for i, s in enumerate(shapes)]
+    max_norm = 1.0 if norm_type == 2.0 else 0.1
+    scaled, total, coef = co.clip_grad_norm(gs, max_norm, norm_type)
+    assert coef < 1.0  # this case clips
+    # (a) in-place clip, as the reference leaves the gradients
+    gws, ggs = [dev(w) for w in ws], [dev(g) for g in gs]
+    opt = ops.MultiTensorAdamW(gws, ggs, t=0, **HYPER)
+    norm = opt.clip_grad_norm_(max_norm, norm_type)
+    assert abs(norm.item() - total) <= 1e-5 * total
+    for i in range(len(shapes)):
+        assert_close(ggs[i], scaled[i], atol=1e-9, name=f"scaled g[{i}]")
+    # (b) the fused form leaves the gradients alone and makes the same update as (a) + plain step
+    gws2, ggs2 = [dev(w) for w in ws], [dev(g) for g in gs]
+    opt2 = ops.MultiTensorAdamW(gws2, ggs2, t=0, **HYPER)
+    norm2 = opt2.step(max_grad_norm=max_norm, norm_type=norm_type)
+    assert norm2.item() == norm.item()  # the same two launches: the same bits
+    opt.step()
+    for i in range(len(shapes)):
+        assert_bit_exact(ggs2[i], gs[i], f"gradient {i} untouched")
+        assert_bit_exact(gws2[i], gws[i], f"fused == clip then step [{i}]")
+        w2, _, _, _ = co.adamw_step(ws[i], scaled[i], torch.zeros_like(ws[i]), torch.zeros_like(ws[i]), t=1, **HYPER)
+        assert_close(gws2[i], w2.reshape(shapes[i]), atol=1e-6, name=f"w[{i}]")
+    # (c) below the threshold nothing changes
+    opt3 = ops.MultiTensorAdamW([dev(w) for w in ws], [dev(g) for g in gs], t=0, **HYPER)
+    opt3.clip_grad_norm_(1e9, norm_type)
+    for i in range(len(shapes)):
+        assert_bit_exact(opt3._grads[i], gs[i], f"no clipping [{i}]")
+
+
+def test_grad_norm_gpt2_small_closed_form(ops):
+    """All 124M gradients equal to c: the 2-norm is c * sqrt(n), the largest magnitude is c."""
+    shapes = gpt2_param_shapes()
+    sizes = [math.prod(s) for s in shapes]
+    total = sum(sizes)
+    flat_w = torch.zeros(total, device=DEV)
+    flat_g = torch.full((total,), 3e-3, device=DEV)
+    offs = [0]
+    for s in sizes:
+        offs.append(offs[-1] + s)
+    opt = ops.MultiTensorAdamW([flat_w[offs[i]:offs[i + 1]] for i in range(len(sizes))],
+                               [flat_g[offs[i]:offs[i + 1]] for i in range(len(sizes))], t=0, **HYPER)
+    c = torch.tensor(3e-3, dtype=torch.float32).item()
+    n2 = opt.grad_norm(1.0, 2.0).item()
+    assert abs(n2 - c * math.sqrt(total)) <= 1e-6 * c * math.sqrt(total)
+    assert abs(opt._clip.item() - 1.0 / (n2 + 1e-6)) <= 1e-6
+    assert opt.grad_norm(1.0, float("inf")).item() == c
+
+
 # ------------------------------------------------------------------- GeLU
 GELU_ATOL = {torch.float32: 1e-6, torch.float64: 1e-14, torch.bfloat16: 1e-6, torch.float16: 1e-6}
 

@@ -355,6 +355,52 @@ def test_adamw_module_matches_torch_optimizer(host, sched):
     assert opt.get_lr() == 5e-3 and all(s.get_lr() == 5e-3 for s in states.values())
 
 
+@pytest.mark.gpu
+def test_clip_grad_norm_task_and_clipped_optimizer(host, sched, co):
+    # Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746) against torch.nn.utils.clip_grad_norm_,
+    # then the module optimizer with max_grad_norm against clip + torch.optim.AdamW
+    shapes = [(300, 64), (64,), (5000,), (17, 3)]
+    gs = [randn(s, 70 + i, std=0.1) for i, s in enumerate(shapes)]
+    handles = [up(host, sched, g.clone()) for g in gs]
+    norm = host.clip_grad_norm_(sched, handles, 0.5, 2.0)
+    ps = [torch.nn.Parameter(torch.zeros(s)) for s in shapes]
+    for p, g in zip(ps, gs):
+        p.grad = g.clone()
+    want = torch.nn.utils.clip_grad_norm_(ps, 0.5, foreach=False)
+    assert abs(down(host, sched, norm).item() - want.item()) <= 1e-5 * want.item()
+    for h, p in zip(handles, ps):
+        assert torch.allclose(down(host, sched, h), p.grad, rtol=1e-5, atol=1e-9)
+
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    root, mods = build_tree(host, sched)
+    opt = host.AdamWModule(sched, root, max_grad_norm=0.05, **hp)
+    assert not opt.last_grad_norm().defined()
+    ref_params = {k: torch.nn.Parameter(down(host, sched, p).clone()) for k, p in root.named_parameters()}
+    ref = torch.optim.AdamW(ref_params.values(), lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"],
+                            weight_decay=hp["weight_decay"], foreach=False)
+    B, T, C = 2, 16, 64
+    used = ("wte.weight", "h.0.ln_1.weight", "h.0.ln_1.bias")
+    for step in range(2):
+        ids = randint(0, 211, (B, T), 80 + step, dtype=torch.int64)
+        y = mods["ln1"].forward(sched, mods["wte"].forward(sched, up(host, sched, ids)))
+        dx = mods["ln1"].backward(sched, up(host, sched, randn((B, T, C), 90 + step)))
+        mods["wte"].backward(sched, dx)
+        grads = dict(root.named_gradients())
+        for k, p in ref_params.items():
+            p.grad = down(host, sched, grads[k]).clone() if k in used else None
+        before = {k: down(host, sched, grads[k]).clone() for k in used}
+        opt.step(sched)
+        want = torch.nn.utils.clip_grad_norm_([ref_params[k] for k in used], 0.05, foreach=False)
+        ref.step()
+        got = down(host, sched, opt.last_grad_norm()).item()
+        assert got > 0.05 and abs(got - want.item()) <= 1e-5 * want.item()
+        for k in used:  # the fused step leaves the gradients as they were
+            assert_bit_exact(down(host, sched, grads[k]), before[k], k)
+        opt.zero_grad(sched)
+    for k, p in root.named_parameters():
+        assert torch.allclose(down(host, sched, p), ref_params[k].detach(), 1e-4, 1e-5), k
+
+
 # ------------------------------------------------------ error conventions (no GPU)
 def run_snippet(code):
     env = dict(os.environ, PYTHONPATH=ROOT)

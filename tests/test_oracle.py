@@ -118,6 +118,34 @@ def test_adamw_f64_agrees_with_f32_and_with_double_brute_force():
 
 
 # ------------------------------------------------------------------- GeLU
+@pytest.mark.parametrize("norm_type", [2.0, float("inf")])
+def test_clip_grad_norm_matches_torch_and_closed_forms(norm_type):
+    # Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746) restates torch.nn.utils.clip_grad_norm_
+    g = [randn((1000,), 1), randn((37, 5), 2), randn((1,), 3)]
+    ps = [torch.nn.Parameter(torch.zeros_like(x)) for x in g]
+    for p, x in zip(ps, g):
+        p.grad = x.clone()
+    ref = torch.nn.utils.clip_grad_norm_(ps, 0.5, norm_type=norm_type, foreach=False)
+    out, total, coef = co.clip_grad_norm(g, 0.5, norm_type)
+    assert abs(total - ref.item()) <= 1e-6 * ref.item()
+    for p, o in zip(ps, out):
+        assert torch.allclose(p.grad, o, rtol=1e-6, atol=0)
+    # closed forms: n copies of c have 2-norm c sqrt(n) and largest magnitude c; the coefficient is
+    # max_norm / (total + 1e-6), and 1 (gradients untouched, bit for bit) when total <= max_norm
+    ones = [torch.full((50,), 2.0), torch.full((14,), -2.0)]
+    out, total, coef = co.clip_grad_norm(ones, 4.0, norm_type)
+    want = 16.0 if norm_type == 2.0 else 2.0
+    assert total == want and abs(coef - min(1.0, 4.0 / (want + 1e-6))) < 1e-7
+    if norm_type == 2.0:
+        assert all(torch.allclose(o, x * 0.25, rtol=1e-6) for o, x in zip(out, ones))
+    out, total, coef = co.clip_grad_norm(g, 1e6, norm_type)
+    assert coef == 1.0 and all(torch.equal(o, x) for o, x in zip(out, g))
+    # a sign error or a dropped tensor would show here: the norm of the concatenation
+    brute = torch.cat([x.flatten().double() for x in g])
+    want = brute.abs().max().item() if norm_type != 2.0 else brute.square().sum().sqrt().item()
+    assert abs(co.clip_grad_norm(g, 1.0, norm_type)[1] - want) <= 1e-6 * want
+
+
 @pytest.mark.parametrize("mode", ["none", "tanh"])
 def test_gelu_matches_aten_cpu(mode):
     x = randn(20000, 11, std=1.5)
