@@ -248,6 +248,22 @@ def per_op_table(args, torch, ops):
         add("layernorm_bwd", f"{tag} [{rows},{C}] bf16", bwd_bytes, mk,
             lambda s: ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma))
 
+        # the residual stream folded into the call (x + residual -> LayerNorm; LayerNorm backward
+        # + dresidual), next to the same work as a separate elementwise add around the plain call
+        def mk_res():
+            st = mk()
+            st["res"] = randn((rows, C))
+            return st
+
+        add("add_layernorm_fwd", f"{tag} [{rows},{C}] bf16, one call", fwd_bytes + 2 * rows * C * 2, mk_res,
+            lambda s: ops.add_layernorm_forward(s["x"], s["res"], gamma, beta, 1e-5))
+        add("add_then_layernorm_fwd", f"{tag} [{rows},{C}] bf16, torch.add + call", fwd_bytes + 2 * rows * C * 2, mk_res,
+            lambda s: ops.layernorm_forward(torch.add(s["x"], s["res"]), gamma, beta, 1e-5))
+        add("layernorm_bwd_add", f"{tag} [{rows},{C}] bf16, one call", bwd_bytes + rows * C * 2, mk_res,
+            lambda s: ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma, dresidual=s["res"]))
+        add("layernorm_bwd_then_add", f"{tag} [{rows},{C}] bf16, call + torch.add", bwd_bytes + rows * C * 2, mk_res,
+            lambda s: torch.add(ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma)[0], s["res"]))
+
     # ---- configuration 3: GeLU [8192,3072] bf16, tanh (benchmark) and erf (the reference's form)
     n = 8192 * 3072
     for mode in ("tanh", "none"):

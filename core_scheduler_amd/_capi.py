@@ -66,6 +66,14 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 6 + [c_int64, c_int64, c_double, c_int, c_int, c_int, c_void_p],
     ),
+    "cs_add_layernorm_forward": (
+        c_int,
+        [c_void_p] * 8 + [c_int64, c_int64, c_double, c_int, c_int, c_int, c_void_p],
+    ),
+    "cs_layernorm_backward_add": (
+        c_int,
+        [c_void_p] * 10 + [c_size_t, c_int64, c_int64] + [c_int] * 5 + [c_void_p],
+    ),
     "cs_layernorm_backward_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "cs_layernorm_backward": (
         c_int,

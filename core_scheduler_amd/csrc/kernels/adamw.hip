@@ -46,7 +46,7 @@ __device__ __forceinline__ void adam_update(T &w, T &m, T &v, T &vmax, const T g
                                             const typename Acc<T>::type gscale) {
   using U = typename Acc<T>::type;
   const U one = (U)1;
-  const U g = to_acc(from_acc<T>(to_acc(g_in) * gscale));
+  const U g = round_through<T>(to_acc(g_in) * gscale);
   const U w0 = to_acc(w);
   const U theta = w0 - h.lr * h.wd * w0;
   const U m_t = h.beta1 * to_acc(m) + (one - h.beta1) * g;

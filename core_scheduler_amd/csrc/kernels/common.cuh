@@ -53,6 +53,11 @@ __device__ __forceinline__ double from_acc<double>(double x) {
 }
 template <>
 __device__ __forceinline__ f16_t from_acc<f16_t>(float x) {
+  // The float result is rounded to half here and nowhere else: without the empty asm the
+  // compiler may merge this conversion into the multiply or add that produced x (one rounding
+  // of the exact result instead of two), which changes ties and makes variants of a kernel
+  // disagree in the last bit.
+  asm volatile("" : "+v"(x));
   f16_t r;
   r.v = (_Float16)x;
   return r;
@@ -62,6 +67,17 @@ __device__ __forceinline__ bf16_t from_acc<bf16_t>(float x) {
   bf16_t r;
   r.bits = f32_to_bf16_bits(x);
   return r;
+}
+
+// x rounded to T's precision and widened again, for arithmetic that must see what a store to
+// T followed by a load would give.
+template <typename T>
+__device__ __forceinline__ typename Acc<T>::type round_through(typename Acc<T>::type x) {
+  return to_acc(from_acc<T>(x));
+}
+template <>
+__device__ __forceinline__ float round_through<f16_t>(float x) {
+  return (float)from_acc<f16_t>(x).v;  // from_acc keeps the conversion a separate rounding
 }
 
 // ------------------------------------------------------- 128-bit vectors

@@ -28,6 +28,11 @@
 
 #include <type_traits>
 
+// Every product and sum below is rounded as written: no multiply-add contraction, so that the
+// template variants of one kernel (with and without the fused residual adds, every output
+// mask) produce the same bits for the same row.
+#pragma clang fp contract(off)
+
 namespace cs_hip {
 namespace {
 
@@ -226,12 +231,16 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
 
 // ----------------------------------------------------------- fast backward
 // Same walk as the forward kernel, with dy and x prefetched one step ahead.
+// HAS_DRES: dx_out = dx + dresidual, the gradient add that follows LayerNorm::backward on the
+// residual stream; dx is rounded to its type first, then the sum, as two kernels would.  Only
+// instantiated for the 2-vectors-per-lane plan: wider rows have no registers left for a third
+// input, and there the add runs as its own launch.
 template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int R, bool HAS_DX,
-          bool HAS_DP>
+          bool HAS_DP, bool HAS_DRES>
 __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
     const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
-    float *__restrict__ partial, int64_t rows, int C) {
+    float *__restrict__ partial, int64_t rows, int C, const TDX *__restrict__ dres) {
   constexpr int VN = Vec16<TX>::n;
   extern __shared__ float lds[];  // [waves per block][C]
   const int lane = threadIdx.x & (kWave - 1);
@@ -270,6 +279,8 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
   for (; row0 < rows; row0 += step) {
     RowSet<TDY, VN, VPL, R> dnxt;
     RowSet<TX, VN, VPL, R> xnxt;
+    RowSet<TDX, VN, VPL, R> rcur;  // this step's dresidual rows, in flight during the reductions
+    if constexpr (HAS_DRES) load_rows<TDX, VN, VPL, R>(rcur, dres, row0, rows, C, nvec, lane);
     float nmu[R], nrs[R];
     const int64_t nrow0 = row0 + step;
     if (nrow0 < rows) {
@@ -320,6 +331,8 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
               const float xh = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
               const float dv = raw_get<TDY, VN>(dcur.v[r][j], k);
               o[k] = rs[r] * (dv * g[j][k] - s1 - xh * s2);
+              if constexpr (HAS_DRES)
+                o[k] = round_through<TDX>(o[k]) + raw_get<TDX, VN>(rcur.v[r][j], k);
             }
             store_n<TDX, VN>(dx + (row0 + r) * C + (int64_t)idx * VN, o);
           }
@@ -402,6 +415,61 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__re
   }
 }
 
+// ------------------------------------------------------ elementwise add
+// out = a + b, one fp32 (fp64) add and one rounding per element; out may be a or b.
+constexpr int kAddUnroll = 2;  // 16-byte vectors per lane, all requested before the first use
+
+template <typename T>
+__global__ __launch_bounds__(kLnThreads) void ew_add_kernel(const T *a, const T *b, T *out, int64_t n,
+                                                            bool vec_ok) {
+  constexpr int VN = Vec16<T>::n;
+  using U = typename Acc<T>::type;
+  constexpr int64_t kChunk = (int64_t)kLnThreads * kAddUnroll * VN;
+  const int64_t begin = (int64_t)blockIdx.x * kChunk;
+  const int64_t end = begin + kChunk < n ? begin + kChunk : n;
+  if (vec_ok && end - begin == kChunk) {
+    Vec16<T> va[kAddUnroll], vb[kAddUnroll];
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+      const int64_t off = begin + ((int64_t)u * kLnThreads + threadIdx.x) * VN;
+      va[u] = load16_stream(a + off);
+      vb[u] = load16_stream(b + off);
+    }
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+      const int64_t off = begin + ((int64_t)u * kLnThreads + threadIdx.x) * VN;
+      Vec16<T> vo;
+#pragma unroll
+      for (int k = 0; k < VN; ++k) vo.e[k] = from_acc<T>((U)(to_acc(va[u].e[k]) + to_acc(vb[u].e[k])));
+      store16(out + off, vo);  // read again by the kernel that follows: keep it cached
+    }
+    return;
+  }
+  for (int64_t i = begin + threadIdx.x; i < end; i += kLnThreads)
+    out[i] = from_acc<T>((U)(to_acc(a[i]) + to_acc(b[i])));
+}
+
+template <typename T>
+int launch_add(const void *a, const void *b, void *out, int64_t n, hipStream_t s) {
+  if (n <= 0) return CS_OK;
+  const bool vec_ok = is_aligned16(a) && is_aligned16(b) && is_aligned16(out);
+  const int64_t blocks = ceil_div(n, (int64_t)kLnThreads * kAddUnroll * Vec16<T>::n);
+  if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  ew_add_kernel<T><<<dim3((unsigned)blocks), dim3(kLnThreads), 0, s>>>((const T *)a, (const T *)b, (T *)out, n,
+                                                                      vec_ok);
+  return launch_status();
+}
+
+int launch_add_dtype(int dtype, const void *a, const void *b, void *out, int64_t n, hipStream_t s) {
+  switch (dtype) {
+    case CS_F32: return launch_add<float>(a, b, out, n, s);
+    case CS_F64: return launch_add<double>(a, b, out, n, s);
+    case CS_F16: return launch_add<f16_t>(a, b, out, n, s);
+    case CS_BF16: return launch_add<bf16_t>(a, b, out, n, s);
+  }
+  return CS_ERR_UNSUPPORTED;
+}
+
 // ------------------------------------------------------------ general path
 // One workgroup per row, any C, any alignment, fp64 included.
 template <typename TX, typename TY, typename TP>
@@ -438,7 +506,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_dx_general_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x,
     const typename Acc<TX>::type *__restrict__ mean,
     const typename Acc<TX>::type *__restrict__ rstd, const TP *__restrict__ gamma,
-    TDX *__restrict__ dx, int64_t C) {
+    TDX *__restrict__ dx, int64_t C, const TDX *__restrict__ dres) {
   using U = typename Acc<TX>::type;
   __shared__ U scratch[kLnThreads / kWave];
   const int64_t row = blockIdx.x;
@@ -455,7 +523,9 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_dx_general_kernel(
   for (int64_t c = threadIdx.x; c < C; c += kLnThreads) {
     const U gd = (U)to_acc(dy[row * C + c]) * (U)to_acc(gamma[c]);
     const U xh = ((U)to_acc(x[row * C + c]) - mu) * rs;
-    dx[row * C + c] = from_acc<TDX>((U)(rs * (gd - s1 - xh * s2)));
+    TDX o = from_acc<TDX>((U)(rs * (gd - s1 - xh * s2)));
+    if (dres) o = from_acc<TDX>((U)(round_through<TDX>((U)to_acc(o)) + (U)to_acc(dres[row * C + c])));
+    dx[row * C + c] = o;
   }
 }
 
@@ -503,6 +573,9 @@ struct FastPlan {
   int fwd_rows = 1;  // rows a wave normalises per step, forward
   int bwd_rows = 1;  // the same, backward (it holds twice the data per row)
 };
+// The widest plan whose backward kernel still has registers for a third input per row
+// (dresidual); wider rows get dx + dresidual from a second launch.
+constexpr int kMaxVplWithResidual = 2;
 
 // x vectors per lane needed for C columns of x_dtype; the fast kernels are
 // instantiated for 2, 4 and 8.
@@ -574,9 +647,14 @@ template <typename TDY, typename TX, typename TDX, typename TP>
 int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
               const void *gamma, void *dx, void *dgamma, void *dbeta, void *workspace,
               size_t workspace_bytes, int64_t rows, int64_t C, bool aligned, int x_dtype,
-              int accumulate, hipStream_t s) {
+              int accumulate, const void *dres, hipStream_t s) {
   const bool want_dp = dgamma != nullptr || dbeta != nullptr;
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
+  // dx + dresidual inside the kernel where it fits (17.5 -> 22 us against 25 us for two
+  // launches at [8192,768] bf16), as a second, in-place launch elsewhere
+  const bool fuse_dres = dres != nullptr && p.vpl != 0 && p.vpl <= kMaxVplWithResidual && is_aligned16(dres);
+  const void *late_dres = fuse_dres ? nullptr : dres;
+  if (!fuse_dres) dres = nullptr;
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
       const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks, kLnBwdThreads);
@@ -584,19 +662,24 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
       const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
       const dim3 grid((unsigned)blocks), block(kLnBwdThreads);
-#define CS_LN_BWD(VPL, R, HAS_DX, HAS_DP)                                                   \
-  ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, R, HAS_DX, HAS_DP><<<grid, block, lds, s>>>(    \
-      (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd,             \
-      (const TP *)gamma, (TDX *)dx, (float *)workspace, rows, (int)C)
+#define CS_LN_BWD(VPL, R, HAS_DX, HAS_DP, HAS_DRES)                                         \
+  ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, R, HAS_DX, HAS_DP, HAS_DRES>                    \
+      <<<grid, block, lds, s>>>((const TDY *)dy, (const TX *)x, (const float *)mean,        \
+                                (const float *)rstd, (const TP *)gamma, (TDX *)dx,          \
+                                (float *)workspace, rows, (int)C, (const TDX *)dres)
 #define CS_LN_BWD_MASK(VPL, R)                \
   if (dx && want_dp) {                        \
-    CS_LN_BWD(VPL, R, true, true);            \
+    CS_LN_BWD(VPL, R, true, true, false);     \
   } else if (dx) {                            \
-    CS_LN_BWD(VPL, R, true, false);           \
+    CS_LN_BWD(VPL, R, true, false, false);    \
   } else {                                    \
-    CS_LN_BWD(VPL, R, false, true);           \
+    CS_LN_BWD(VPL, R, false, true, false);    \
   }
-      if (p.vpl == 2) {
+      if (p.vpl == 2 && dres && want_dp) {
+        CS_LN_BWD(2, CS_LN_BWD_ROWS_VPL2, true, true, true);
+      } else if (p.vpl == 2 && dres) {
+        CS_LN_BWD(2, CS_LN_BWD_ROWS_VPL2, true, false, true);
+      } else if (p.vpl == 2) {
         CS_LN_BWD_MASK(2, CS_LN_BWD_ROWS_VPL2)
       } else if (p.vpl == 4) {
         CS_LN_BWD_MASK(4, CS_LN_BWD_ROWS_VPL4)
@@ -606,10 +689,13 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
 #undef CS_LN_BWD_MASK
 #undef CS_LN_BWD
       int st = launch_status();
-      if (st != CS_OK || !want_dp) return st;
-      ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
-          (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, accumulate);
-      return launch_status();
+      if (st == CS_OK && want_dp) {
+        ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
+            (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, accumulate);
+        st = launch_status();
+      }
+      if (st == CS_OK && late_dres) st = launch_add<TDX>(dx, late_dres, dx, rows * C, s);
+      return st;
     }
   }
   using U = typename Acc<TX>::type;
@@ -617,7 +703,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   if (dx) {
     ln_bwd_dx_general_kernel<TDY, TX, TDX, TP><<<dim3((unsigned)rows), dim3(kLnThreads), 0, s>>>(
         (const TDY *)dy, (const TX *)x, (const U *)mean, (const U *)rstd, (const TP *)gamma,
-        (TDX *)dx, C);
+        (TDX *)dx, C, (const TDX *)late_dres);
     const int st = launch_status();
     if (st != CS_OK) return st;
   }
@@ -638,9 +724,10 @@ bool wide_ok(int narrow, int other) { return other == narrow || other == CS_F32;
 
 using namespace cs_hip;
 
-extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void *beta, void *y,
-                                    void *mean, void *rstd, int64_t rows, int64_t C, double eps,
-                                    int x_dtype, int y_dtype, int param_dtype, void *stream) {
+namespace {
+int ln_forward(const void *x, const void *residual, void *sum_out, const void *gamma,
+               const void *beta, void *y, void *mean, void *rstd, int64_t rows, int64_t C,
+               double eps, int x_dtype, int y_dtype, int param_dtype, void *stream) {
   if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
   if (dtype_size(x_dtype) == 0 || dtype_size(y_dtype) == 0 || dtype_size(param_dtype) == 0)
     return CS_ERR_UNSUPPORTED;
@@ -648,14 +735,25 @@ extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void
   if (x_dtype == CS_F64 && (y_dtype != CS_F64 || param_dtype != CS_F64)) return CS_ERR_UNSUPPORTED;
   if (rows == 0) return CS_OK;
   if (!x || !gamma || !y || !mean || !rstd) return CS_ERR_INVALID_ARGUMENT;
+  if ((residual == nullptr) != (sum_out == nullptr)) return CS_ERR_INVALID_ARGUMENT;
+  if (residual && (!aligned_to(residual, dtype_size(x_dtype)) || !aligned_to(sum_out, dtype_size(x_dtype))))
+    return CS_ERR_MISALIGNED;
   if (!aligned_to(x, dtype_size(x_dtype)) || !aligned_to(y, dtype_size(y_dtype)) ||
       !aligned_to(gamma, dtype_size(param_dtype)) ||
       (beta && !aligned_to(beta, dtype_size(param_dtype))) || !aligned_to(mean, 4) ||
       !aligned_to(rstd, 4))
     return CS_ERR_MISALIGNED;
-  const bool aligned =
-      is_aligned16(x) && is_aligned16(y) && is_aligned16(gamma) && (!beta || is_aligned16(beta));
+  const bool aligned = is_aligned16(residual ? sum_out : x) && is_aligned16(y) &&
+                       is_aligned16(gamma) && (!beta || is_aligned16(beta));
   hipStream_t s = as_stream(stream);
+  if (residual) {
+    // Measured on MI355X, [8192,768] and [16384,1600] bf16: the sum written by an add launch is
+    // still in the last-level cache when the normalising launch reads it, and the two launches
+    // (17 / 47 us) beat one kernel with two input and two output streams per row (20 / 52 us).
+    const int st = launch_add_dtype(x_dtype, x, residual, sum_out, rows * C, s);
+    if (st != CS_OK) return st;
+    x = sum_out;
+  }
 #define CS_CALL(TX, TY, TP) \
   return fwd_typed<TX, TY, TP>(x, gamma, beta, y, mean, rstd, rows, C, eps, aligned, x_dtype, s)
   const bool y_wide = y_dtype != x_dtype, p_wide = param_dtype != x_dtype;
@@ -676,6 +774,23 @@ extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void
 #undef CS_CALL
   return CS_ERR_UNSUPPORTED;
 }
+}  // namespace
+
+extern "C" int cs_layernorm_forward(const void *x, const void *gamma, const void *beta, void *y,
+                                    void *mean, void *rstd, int64_t rows, int64_t C, double eps,
+                                    int x_dtype, int y_dtype, int param_dtype, void *stream) {
+  return ln_forward(x, nullptr, nullptr, gamma, beta, y, mean, rstd, rows, C, eps, x_dtype, y_dtype,
+                    param_dtype, stream);
+}
+
+extern "C" int cs_add_layernorm_forward(const void *x, const void *residual, void *sum_out,
+                                        const void *gamma, const void *beta, void *y, void *mean,
+                                        void *rstd, int64_t rows, int64_t C, double eps,
+                                        int x_dtype, int y_dtype, int param_dtype, void *stream) {
+  if (rows > 0 && (!residual || !sum_out)) return CS_ERR_INVALID_ARGUMENT;
+  return ln_forward(x, residual, sum_out, gamma, beta, y, mean, rstd, rows, C, eps, x_dtype, y_dtype,
+                    param_dtype, stream);
+}
 
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
@@ -683,11 +798,11 @@ extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C)
   return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads) * 2 * (size_t)C * sizeof(float);
 }
 
-extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
-                                     const void *rstd, const void *gamma, void *dx, void *dgamma,
-                                     void *dbeta, void *workspace, size_t workspace_bytes,
-                                     int64_t rows, int64_t C, int dy_dtype, int x_dtype,
-                                     int dx_dtype, int param_dtype, int accumulate, void *stream) {
+namespace {
+int ln_backward(const void *dy, const void *x, const void *mean, const void *rstd,
+                const void *gamma, const void *dres, void *dx, void *dgamma, void *dbeta,
+                void *workspace, size_t workspace_bytes, int64_t rows, int64_t C, int dy_dtype,
+                int x_dtype, int dx_dtype, int param_dtype, int accumulate, void *stream) {
   if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
   if (dtype_size(x_dtype) == 0 || dtype_size(dy_dtype) == 0 || dtype_size(dx_dtype) == 0 ||
       dtype_size(param_dtype) == 0)
@@ -703,6 +818,8 @@ extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *
     return CS_OK;
   }
   if (!dy || !x || !mean || !rstd || (dx && !gamma)) return CS_ERR_INVALID_ARGUMENT;
+  if (dres && !dx) return CS_ERR_INVALID_ARGUMENT;
+  if (dres && !aligned_to(dres, dtype_size(dx_dtype))) return CS_ERR_MISALIGNED;
   if (!aligned_to(dy, dtype_size(dy_dtype)) || !aligned_to(x, dtype_size(x_dtype)) ||
       (dx && !aligned_to(dx, dtype_size(dx_dtype))) ||
       (gamma && !aligned_to(gamma, dtype_size(param_dtype))) ||
@@ -711,11 +828,12 @@ extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *
       !aligned_to(rstd, 4))
     return CS_ERR_MISALIGNED;
   const bool aligned = is_aligned16(dy) && is_aligned16(x) && (!dx || is_aligned16(dx)) &&
-                       (!dx || is_aligned16(gamma)) && (!workspace || is_aligned16(workspace));
+                       (!dx || is_aligned16(gamma)) && (!workspace || is_aligned16(workspace)) &&
+                       (!dres || is_aligned16(dres));
   hipStream_t s = as_stream(stream);
 #define CS_CALL(TDY, TX, TDX, TP)                                                              \
   return bwd_typed<TDY, TX, TDX, TP>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, workspace,   \
-                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, s)
+                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, dres, s)
   const bool dy_wide = dy_dtype != x_dtype, dx_wide = dx_dtype != x_dtype,
              p_wide = param_dtype != x_dtype;
   switch (x_dtype) {
@@ -735,4 +853,27 @@ extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *
   }
 #undef CS_CALL
   return CS_ERR_UNSUPPORTED;
+}
+}  // namespace
+
+extern "C" int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
+                                     const void *rstd, const void *gamma, void *dx, void *dgamma,
+                                     void *dbeta, void *workspace, size_t workspace_bytes,
+                                     int64_t rows, int64_t C, int dy_dtype, int x_dtype,
+                                     int dx_dtype, int param_dtype, int accumulate, void *stream) {
+  return ln_backward(dy, x, mean, rstd, gamma, nullptr, dx, dgamma, dbeta, workspace, workspace_bytes,
+                     rows, C, dy_dtype, x_dtype, dx_dtype, param_dtype, accumulate, stream);
+}
+
+extern "C" int cs_layernorm_backward_add(const void *dy, const void *x, const void *mean,
+                                         const void *rstd, const void *gamma,
+                                         const void *dresidual, void *dx, void *dgamma,
+                                         void *dbeta, void *workspace, size_t workspace_bytes,
+                                         int64_t rows, int64_t C, int dy_dtype, int x_dtype,
+                                         int dx_dtype, int param_dtype, int accumulate,
+                                         void *stream) {
+  if (rows > 0 && (!dresidual || !dx)) return CS_ERR_INVALID_ARGUMENT;
+  return ln_backward(dy, x, mean, rstd, gamma, dresidual, dx, dgamma, dbeta, workspace,
+                     workspace_bytes, rows, C, dy_dtype, x_dtype, dx_dtype, param_dtype, accumulate,
+                     stream);
 }

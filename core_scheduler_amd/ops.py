@@ -185,6 +185,28 @@ def gelu_backward(dy, x, approximate="none"):
 
 
 # -------------------------------------------------------------- LayerNorm
+def add_layernorm_forward(x, residual, gamma, beta=None, eps=1e-5, out_dtype=None, inplace=False):
+    """s = x + residual; returns (s, LayerNorm(s), mean, rstd) from one pass.  `inplace` writes s over x."""
+    dev = _dev(x, residual, gamma, beta)
+    if residual.shape != x.shape or residual.dtype != x.dtype:
+        raise ValueError("residual must match x")
+    C = x.shape[-1]
+    rows = x.numel() // C
+    if gamma.numel() != C or (beta is not None and (beta.numel() != C or beta.dtype != gamma.dtype)):
+        raise ValueError("gamma/beta must be [C] of one dtype")
+    total = x if inplace else torch.empty_like(x)
+    y = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=dev)
+    stat = torch.float64 if x.dtype == torch.float64 else torch.float32
+    mean = torch.empty(rows, dtype=stat, device=dev)
+    rstd = torch.empty(rows, dtype=stat, device=dev)
+    with torch.cuda.device(dev):
+        code = _capi.load().cs_add_layernorm_forward(_ptr(x), _ptr(residual), _ptr(total), _ptr(gamma), _ptr(beta),
+                                                     _ptr(y), _ptr(mean), _ptr(rstd), rows, C, eps, _dt(x),
+                                                     _dt(y), _dt(gamma), _stream(dev))
+    _capi.check("cs_add_layernorm_forward", code)
+    return total, y, mean, rstd
+
+
 def layernorm_forward(x, gamma, beta=None, eps=1e-5, out_dtype=None):
     """Returns (y, mean, rstd); mean and rstd are [rows] fp32 (fp64 for fp64 x)."""
     dev = _dev(x, gamma, beta)
@@ -205,9 +227,13 @@ def layernorm_forward(x, gamma, beta=None, eps=1e-5, out_dtype=None):
 
 
 def layernorm_backward(dy, x, mean, rstd, gamma, *, need_dx=True, need_dgamma=True, need_dbeta=True,
-                       dgamma=None, dbeta=None, dx_dtype=None):
-    """Returns (dx, dgamma, dbeta).  Passing dgamma / dbeta accumulates into them."""
-    dev = _dev(dy, x, mean, rstd, gamma, dgamma, dbeta)
+                       dgamma=None, dbeta=None, dx_dtype=None, dresidual=None):
+    """Returns (dx, dgamma, dbeta).  Passing dgamma / dbeta accumulates into them; `dresidual`
+    (same shape and dtype as dx) is added to dx in the same pass."""
+    dev = _dev(dy, x, mean, rstd, gamma, dgamma, dbeta, dresidual)
+    if dresidual is not None and (not need_dx or dresidual.shape != x.shape
+                                  or dresidual.dtype != (dx_dtype or x.dtype)):
+        raise ValueError("dresidual must match dx")
     C = x.shape[-1]
     rows = x.numel() // C
     accumulate = dgamma is not None or dbeta is not None
@@ -226,10 +252,16 @@ def layernorm_backward(dy, x, mean, rstd, gamma, *, need_dx=True, need_dgamma=Tr
     ws_bytes = lib.cs_layernorm_backward_workspace_bytes(rows, C) if (need_dgamma or need_dbeta) else 0
     ws = _workspace(ws_bytes, dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        code = lib.cs_layernorm_backward(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma), _ptr(dx),
-                                         _ptr(dgamma), _ptr(dbeta), _ptr(ws), ws_bytes, rows, C, _dt(dy),
-                                         _dt(x), _dt(dx) if dx is not None else _dt(x), _dt(gamma),
-                                         int(accumulate), _stream(dev))
+        if dresidual is not None:
+            code = lib.cs_layernorm_backward_add(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma),
+                                                 _ptr(dresidual), _ptr(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws),
+                                                 ws_bytes, rows, C, _dt(dy), _dt(x), _dt(dx), _dt(gamma),
+                                                 int(accumulate), _stream(dev))
+        else:
+            code = lib.cs_layernorm_backward(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma), _ptr(dx),
+                                             _ptr(dgamma), _ptr(dbeta), _ptr(ws), ws_bytes, rows, C, _dt(dy),
+                                             _dt(x), _dt(dx) if dx is not None else _dt(x), _dt(gamma),
+                                             int(accumulate), _stream(dev))
     _capi.check("cs_layernorm_backward", code)
     return dx, dgamma, dbeta
 

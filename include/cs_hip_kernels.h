@@ -195,6 +195,31 @@ int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
                           int dy_dtype, int x_dtype, int dx_dtype,
                           int param_dtype, int accumulate, void *stream);
 
+/* The residual stream around LayerNorm, fused (the transformer block of
+ * example/gpt2/gpt2_single_device.cpp:457-464 and :467-474):
+ *   forward : sum_out = x + residual;  y = LayerNorm(sum_out)
+ *             replaces Utils::add (:459) followed by ln2->forward (:460)
+ *   backward: dx = LayerNorm_backward(dy) + dresidual
+ *             replaces ln2->backward (:468) followed by Utils::add (:469)
+ * Each removes one [rows, C] round trip.  Results are those of the two
+ * separate kernels: the sum is rounded to x_dtype before it is normalised,
+ * and dx is rounded to dx_dtype before dresidual is added.  residual and
+ * sum_out are [rows, C] of x_dtype (sum_out may be x or residual itself);
+ * dresidual is [rows, C] of dx_dtype (dx may be dresidual itself).  All other
+ * arguments as in the plain calls. */
+int cs_add_layernorm_forward(const void *x, const void *residual,
+                             void *sum_out, const void *gamma,
+                             const void *beta, void *y, void *mean, void *rstd,
+                             int64_t rows, int64_t C, double eps, int x_dtype,
+                             int y_dtype, int param_dtype, void *stream);
+int cs_layernorm_backward_add(const void *dy, const void *x, const void *mean,
+                              const void *rstd, const void *gamma,
+                              const void *dresidual, void *dx, void *dgamma,
+                              void *dbeta, void *workspace,
+                              size_t workspace_bytes, int64_t rows, int64_t C,
+                              int dy_dtype, int x_dtype, int dx_dtype,
+                              int param_dtype, int accumulate, void *stream);
+
 /* ------------------------------------------------------------------------
  * Embedding
  * forward replaces torch::embedding, src/compute/embedding.cpp:117-121:

@@ -153,7 +153,7 @@ def test_adamw_gpt2_small_ten_steps(ops, co):
 
 
 @pytest.mark.parametrize("norm_type", [2.0, float("inf")])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_clip_grad_norm_and_clipped_step(ops, co, norm_type, dtype):
     """Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746): norm, coefficient, in-place scaling,
     and the step that applies the coefficient while it reads the gradients."""
@@ -287,6 +287,73 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
 ])
 def test_layernorm(ops, co, rows, C, x_dtype, p_dtype):
     _ln_case(ops, co, rows, C, x_dtype, p_dtype)
+
+
+@pytest.mark.parametrize("rows,C,x_dtype,p_dtype", [
+    (8192, 768, torch.bfloat16, torch.float32),     # benchmark configuration 3
+    (2048, 1600, torch.bfloat16, torch.float32),    # XL width
+    (1024, 384, torch.float32, torch.float32),
+    (513, 768, torch.float16, torch.float16),
+    (77, 4096, torch.bfloat16, torch.float32),      # 8 vectors per lane plan
+    (5, 768, torch.float32, torch.float32),
+    (64, 50, torch.float32, torch.float32),         # general path
+    (33, 10000, torch.bfloat16, torch.float32),     # general path
+    (128, 384, torch.float64, torch.float64),
+])
+def test_layernorm_with_residual_stream(ops, co, rows, C, x_dtype, p_dtype):
+    """x + residual -> LayerNorm, and LayerNorm backward + dresidual, each in one pass
+    (example/gpt2/gpt2_single_device.cpp:459-460 and :468-469).  The fused results must be the
+    bits of the separate kernels, and agree with the oracle applied to the rounded sum."""
+    x = randn((rows, C), 60, dtype=x_dtype)
+    res = randn((rows, C), 61, dtype=x_dtype)
+    gamma = randn(C, 62, std=0.02, mean=1.0, dtype=p_dtype)
+    beta = randn(C, 63, std=0.02, dtype=p_dtype)
+    dy = randn((rows, C), 64, dtype=x_dtype)
+    dres = randn((rows, C), 65, dtype=x_dtype)
+    gx, gres, gg, gb = dev(x), dev(res), dev(gamma), dev(beta)
+    total, y, mean, rstd = ops.add_layernorm_forward(gx, gres, gg, gb, 1e-5)
+    wide = torch.float64 if x_dtype == torch.float64 else torch.float32
+    total_ref = (x.to(wide) + res.to(wide)).to(x_dtype)   # one add, one rounding
+    assert_bit_exact(total, total_ref, "x + residual")
+    y_sep, mean_sep, rstd_sep = ops.layernorm_forward(dev(total_ref), gg, gb, 1e-5)
+    # rows of 5 to 8 vectors per lane run the register-resident kernel only without a residual,
+    # so there the two results come from different summation orders
+    vec_per_lane = -(-C * x.element_size() // 16 // 64)
+    same_kernel = not (4 < vec_per_lane <= 8 and C * x.element_size() % 16 == 0 and x_dtype != torch.float64)
+    same = assert_bit_exact if same_kernel else (lambda a, b, name: assert_close(a, b, atol=2e-6, name=name))
+    same(y, y_sep, "y: fused == separate kernels")
+    same(mean, mean_sep, "mean")
+    same(rstd, rstd_sep, "rstd")
+    y2, mean2, rstd2 = co.layernorm_forward(total_ref, gamma, beta, 1e-5)
+    assert_close(y, y2, atol=2e-6, name="y vs oracle")
+    assert_close(rstd, rstd2, atol=1e-6, name="rstd vs oracle")
+    # in place: the sum lands in x's buffer
+    gx2 = dev(x).clone()
+    t2, y_ip, _, _ = ops.add_layernorm_forward(gx2, gres, gg, gb, 1e-5, inplace=True)
+    assert t2.data_ptr() == gx2.data_ptr()
+    assert_bit_exact(gx2, total_ref, "in-place sum")
+    assert_bit_exact(y_ip, y, "in-place y")
+    # backward
+    gdy, gdres, gm, gr = dev(dy), dev(dres), dev(mean2), dev(rstd2)
+    dx, dg, db = ops.layernorm_backward(gdy, dev(total_ref), gm, gr, gg, dresidual=gdres)
+    dx_sep, dg_sep, db_sep = ops.layernorm_backward(gdy, dev(total_ref), gm, gr, gg)
+    want = (dx_sep.to(wide) + gdres.to(wide)).to(x_dtype)
+    if same_kernel:
+        assert_bit_exact(dx, want, "dx: fused == separate kernels")
+        assert_bit_exact(dg, dg_sep, "dgamma")
+        assert_bit_exact(db, db_sep, "dbeta")
+    # against the oracle: dx itself is held to one unit in the last place of dx, and that unit can
+    # be several units of a smaller sum, so the bound is taken at the size of the terms
+    dx2, _, _ = co.layernorm_backward(dy, total_ref, mean2, rstd2, gamma)
+    want2 = dx2.to(wide) + dres.to(wide)
+    unit = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5, torch.float64: 1e-12}[x_dtype]
+    err = (dx.cpu().to(wide) - want2).abs()
+    bound = unit * (dx2.to(wide).abs() + want2.abs()) + 5e-6
+    assert (err <= bound).all(), f"dx vs oracle: max excess {(err - bound).max().item():.3e}"
+    only_dx, none_g, none_b = ops.layernorm_backward(gdy, dev(total_ref), gm, gr, gg, need_dgamma=False,
+                                                     need_dbeta=False, dresidual=gdres)
+    assert none_g is None and none_b is None
+    assert_bit_exact(only_dx, dx, "dx with mask {1,0,0}")
 
 
 def test_layernorm_without_bias(ops, co):
