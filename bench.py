@@ -300,6 +300,7 @@ def per_op_table(args, torch, ops):
 
     # ---- configuration 0 / 4: AdamW over the GPT-2-small / XL parameter sets, one launch
     for tag, n_layer, C in (("small", 12, 768), ("xl", 48, 1600)):
+        torch.cuda.empty_cache()  # fresh, unfragmented blocks for the four large parameter-sized buffers
         sizes = gpt2_param_sizes(n_layer, C)
         total = sum(sizes)
         if (tag == "xl" and not args.xl_adamw) or not wanted("adamw"):

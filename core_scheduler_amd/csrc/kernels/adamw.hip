@@ -249,18 +249,36 @@ __global__ __launch_bounds__(1024) void grad_norm_final_kernel(const float *__re
                                                                float *__restrict__ clip) {
   __shared__ double scratch[1024 / kWave];
   const int tid = threadIdx.x;
-  // thread t owns the contiguous run of slots [t*per, (t+1)*per): a fixed order
-  const int64_t per = (n_slots + 1023) / 1024;
-  const int64_t lo = (int64_t)tid * per;
-  const int64_t hi = lo + per < n_slots ? lo + per : n_slots;
-  double acc = 0.;
-  for (int64_t i = lo; i < hi; ++i) {
+  // thread t adds slots t, t + 1024, ... (coalesced reads) into four interleaved sums, so four
+  // loads are in flight; the order is fixed, whatever the scheduling
+  double a4[4] = {0., 0., 0., 0.};
+  int64_t i = tid;
+  for (; i + 3 * 1024 < n_slots; i += 4 * 1024) {
+    const float p0 = partial[i], p1 = partial[i + 1024], p2 = partial[i + 2048], p3 = partial[i + 3072];
+    const float p[4] = {p0, p1, p2, p3};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if constexpr (INF) {
+        a4[u] = (double)p[u] > a4[u] ? (double)p[u] : a4[u];
+      } else {
+        a4[u] += (double)p[u];
+      }
+    }
+  }
+  for (; i < n_slots; i += 1024) {
     const double p = (double)partial[i];
     if constexpr (INF) {
-      acc = p > acc ? p : acc;
+      a4[0] = p > a4[0] ? p : a4[0];
     } else {
-      acc += p;
+      a4[0] += p;
     }
+  }
+  double acc;
+  if constexpr (INF) {
+    const double m01 = a4[0] > a4[1] ? a4[0] : a4[1], m23 = a4[2] > a4[3] ? a4[2] : a4[3];
+    acc = m01 > m23 ? m01 : m23;
+  } else {
+    acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
   }
   double total;
   if constexpr (INF) {
