@@ -26,17 +26,6 @@ def load(name):
     return out
 
 
-class Oracle:
-    """Adapter with the same call shapes for the C oracle and the HIP ops."""
-
-    def __init__(self, mod, to):
-        self.m, self.to = mod, to
-
-    def ce(self, x, t, V, **kw):
-        fn = getattr(self.m, "cross_entropy", None) or self.m.fused_classifier
-        return fn(self.to(x), self.to(t), V, **kw)
-
-
 def backends():
     from oracle import c_oracle
 
