@@ -593,3 +593,88 @@ def test_cross_entropy_config2_full_size(ops, co):
     _, row2, d2, _ = co.cross_entropy(x[pick], t[pick], V, reduction="sum", dloss=1.0 / N)
     assert_close(row[pick], row2.float(), atol=1e-5, name="row loss sample")
     assert_close(gx[pick], d2, atol=1e-10, name="dlogits sample")
+
+
+# ------------------------------------------------ configuration 4: GPT-2-XL scale
+def test_xl_cross_entropy(ops, co):
+    """[16384, 50257] bf16, stride 50304: size-independent properties + the oracle on a sample of rows."""
+    N, V, stride = 16384, 50257, 50304
+    g = torch.Generator(device=DEV).manual_seed(1341)
+    gx = (torch.randn((N, stride), generator=g, device=DEV) * 2.0).to(torch.bfloat16)
+    t = randint(0, V, (N,), 1342)
+    pick = torch.arange(0, N, 331)
+    x_pick = gx[pick].cpu()
+    loss, row, d, tw = ops.fused_classifier(gx, dev(t), V, inplace=True)
+    assert tw.item() == N
+    assert (gx[:, V:] == 0).all()
+    assert gx[:, :V].float().sum(1).abs().max().item() < 2e-6
+    assert abs(loss.item() - row.double().mean().item()) < 1e-5
+    assert (gx[torch.arange(N), dev(t)] < 0).all()
+    _, row2, d2, _ = co.cross_entropy(x_pick, t[pick], V, reduction="sum", dloss=1.0 / N)
+    assert_close(row[pick], row2.float(), atol=1e-5, name="row loss sample")
+    assert_close(gx[pick], d2, atol=1e-10, name="dlogits sample")
+
+
+def test_xl_embedding(ops, co):
+    """wte 50257x1600, wpe 1024x1600 bf16, B 16, T 1024, Zipf ids: the whole case against the oracle."""
+    V, C, B, T = 50257, 1600, 16, 1024
+    wte, wpe = randn((V, C), 1343, std=0.02, dtype=torch.bfloat16), randn((T, C), 1344, std=0.02, dtype=torch.bfloat16)
+    ids = zipf_ids(B * T, V, 1345).reshape(B, T)
+    dout = randn((B, T, C), 1346, dtype=torch.bfloat16)
+    assert_bit_exact(ops.embedding_forward_add(dev(wte), dev(wpe), dev(ids)), co.embedding_forward_add(wte, wpe, ids),
+                     "gather-add")
+    dwte, dwpe = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_close(dwte, co.embedding_backward(dout, ids, V), atol=1e-6, name="dwte")
+    assert_close(dwpe, co.embedding_backward_positions(dout), atol=1e-6, name="dwpe")
+    # column sums of the dense gradient equal column sums of dout (nothing dropped, nothing doubled)
+    want = dout.double().sum((0, 1))
+    got = dwte.double().sum(0).cpu()
+    assert (got - want).abs().max().item() < 0.05 * B * T ** 0.5  # bf16 rounding of each output row
+    untouched = torch.ones(V, dtype=torch.bool)
+    untouched[ids.flatten()] = False
+    assert (dwte[dev(untouched)] == 0).all()
+    again = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_bit_exact(again[0], dwte, "dwte rerun")
+
+
+def test_xl_layernorm(ops, co):
+    """[16384, 1600] bf16 with fp32 parameters: forward and backward against the oracle."""
+    _ln_case(ops, co, 16384, 1600, torch.bfloat16, torch.float32)
+
+
+def test_xl_adamw(ops, co):
+    """All 580 GPT-2-XL tensors (1,557,611,200 fp32 parameters) in one launch, two steps; the oracle
+    runs on a sample of tensors (the largest, the smallest, some from the middle and the last)."""
+    shapes = gpt2_param_shapes(48, 1600)
+    sizes = [math.prod(s) for s in shapes]
+    total = sum(sizes)
+    assert len(shapes) == 580 and total == 1_557_611_200
+    g = torch.Generator(device=DEV).manual_seed(1347)
+    w = torch.empty(total, device=DEV).normal_(0, 0.02, generator=g)
+    grad = torch.empty(total, device=DEV).normal_(0, 1e-3, generator=g)
+    offs = [0]
+    for s in sizes:
+        offs.append(offs[-1] + s)
+    sample = [0, 1, 2, 4, 5, 300, 301, 575, 578, 579]
+    w0 = {i: w[offs[i]:offs[i + 1]].cpu() for i in sample}
+    grads = []
+    opt = ops.MultiTensorAdamW([w[offs[i]:offs[i + 1]] for i in range(len(sizes))],
+                               [grad[offs[i]:offs[i + 1]] for i in range(len(sizes))], t=0, **HYPER)
+    for step in range(2):
+        if step == 1:
+            grad.normal_(0, 1e-3, generator=g)
+        grads.append({i: grad[offs[i]:offs[i + 1]].cpu() for i in sample})
+        opt.step()
+    for i in sample:
+        ww, m, v = w0[i], torch.zeros(sizes[i]), torch.zeros(sizes[i])
+        for t in (1, 2):
+            ww, m, v, _ = co.adamw_step(ww, grads[t - 1][i], m, v, t=t, **HYPER)
+        assert_close(w[offs[i]:offs[i + 1]], ww, atol=1e-8, name=f"w[{i}]")
+        assert_close(opt.m[i].flatten(), m, atol=1e-10, name=f"m[{i}]")
+        assert_close(opt.v[i].flatten(), v, atol=1e-13, name=f"v[{i}]")
+    # no element outside the sample was skipped: after two steps from m = 0 with these hyper-parameters
+    # every first moment is non-zero wherever the gradients are, and they are everywhere
+    m_all = torch.cat([x.flatten() for x in opt.m[3:4]])
+    assert (m_all != 0).all()
+    del opt, w, grad
+    torch.cuda.empty_cache()
