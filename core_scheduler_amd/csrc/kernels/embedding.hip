@@ -456,11 +456,17 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
       } else {
         // part of a run that spans waves: slot 1 if it reaches this wave's last entry
         const int slot = e == kOwn - 1 ? 1 : 0;
-        float *dst = lds + (wave * 2 + slot) * kChunkCols;
+        // four columns per 16-byte LDS word; word (j*H + h)*64 + lane holds columns
+        // (lane + 64 j)*VN + 4h .. + 3, so the lanes of a wave write consecutive words
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        constexpr int H = VN / 4;
+        f32x4 *dst = reinterpret_cast<f32x4 *>(lds) + (wave * 2 + slot) * (kChunkCols / 4);
 #pragma unroll
         for (int j = 0; j < kVpl; ++j)
 #pragma unroll
-          for (int k = 0; k < VN; ++k) dst[(lane + kWave * j) * VN + k] = acc[j][k];
+          for (int h = 0; h < H; ++h)
+            dst[(j * H + h) * kWave + lane] =
+                f32x4{acc[j][4 * h], acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]};
       }
     }
     __syncthreads();
@@ -486,7 +492,7 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
         float *prow = partial + (w * 2 + (seg_ends ? 0 : 1)) * C;
         typedef float f32x4 __attribute__((ext_vector_type(4)));
         const f32x4 *lds4 = reinterpret_cast<const f32x4 *>(lds);
-        constexpr int kSlices = kChunkCols / 4 / kWave;  // groups of four columns per lane
+        constexpr int kSlices = kChunkCols / 4 / kWave;  // groups of four columns per lane (kVpl * VN / 4)
         f32x4 t[kSlices];
 #pragma unroll
         for (int v = 0; v < kSlices; ++v) t[v] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -502,8 +508,10 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
         }
 #pragma unroll
         for (int v = 0; v < kSlices; ++v) {
-          const int64_t col = (int64_t)cb * VN + (int64_t)(lane + kWave * v) * 4;
-          if (col >= C) continue;  // C is a multiple of four columns here
+          // slice v = j*H + h of the layout above
+          constexpr int H = VN / 4;
+          const int64_t col = ((int64_t)cb + lane + kWave * (v / H)) * VN + 4 * (v % H);
+          if (col >= C) continue;  // C is a multiple of VN columns here
           if (whole) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {

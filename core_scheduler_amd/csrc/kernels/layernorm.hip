@@ -349,7 +349,9 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
   }
 
   if constexpr (HAS_DP) {
-    // fold the block's waves, dgamma first, then dbeta through the same LDS
+    // fold the block's waves, dgamma first, then dbeta through the same LDS.  Column
+    // idx*VN + k is kept at position k*nvec + idx, in the LDS and in the partial rows: lanes
+    // then write consecutive words (no bank conflicts); the last kernel undoes the permutation.
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
 #pragma unroll
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
         if (idx < nvec) {
 #pragma unroll
           for (int k = 0; k < VN; ++k)
-            lds[wave * C + idx * VN + k] = which == 0 ? acc_g[j][k] : acc_b[j][k];
+            lds[wave * C + k * nvec + idx] = which == 0 ? acc_g[j][k] : acc_b[j][k];
         }
       }
       __syncthreads();
@@ -373,7 +375,8 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
   }
 }
 
-// Adds `nparts` partial rows in a fixed order.  grid (ceil(C/64), 2), block
+// Adds `nparts` partial rows in a fixed order.  Partial rows are permuted: position
+// p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  grid (ceil(C/64), 2), block
 // (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one column
 // into four interleaved accumulators (so four loads are always in flight),
 // then row 0 of the block adds the 16 sub-sums in order.
@@ -381,12 +384,12 @@ template <typename TP>
 __global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__restrict__ partial,
                                                                int nparts, TP *__restrict__ dgamma,
                                                                TP *__restrict__ dbeta, int C,
-                                                               int accumulate) {
+                                                               int vn, int accumulate) {
   __shared__ float sub[16][64];
   const int which = blockIdx.y;
   TP *out = which == 0 ? dgamma : dbeta;
   if (out == nullptr) return;  // block-uniform
-  const int col = blockIdx.x * 64 + threadIdx.x;
+  const int col = blockIdx.x * 64 + threadIdx.x;  // a position in the permuted row
   float s = 0.f;
   if (col < C) {
     const float *src = partial + (int64_t)which * C + col;
@@ -410,8 +413,10 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__re
     float t = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t += sub[r][threadIdx.x];
-    if (accumulate) t += to_acc(out[col]);
-    out[col] = from_acc<TP>(t);
+    const int nvec = C / vn;
+    const int real = (col % nvec) * vn + col / nvec;  // the column this position stands for
+    if (accumulate) t += to_acc(out[real]);
+    out[real] = from_acc<TP>(t);
   }
 }
 
@@ -691,7 +696,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
       int st = launch_status();
       if (st == CS_OK && want_dp) {
         ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
-            (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, accumulate);
+            (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
         st = launch_status();
       }
       if (st == CS_OK && late_dres) st = launch_add<TDX>(dx, late_dres, dx, rows * C, s);
