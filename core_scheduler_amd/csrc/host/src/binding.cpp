@@ -1,6 +1,7 @@
 // Python binding of the host API, so that the parity tests can drive cs::compute /
 // cs::optimizer exactly as the reference's gtest suites do: build a DynamicScheduler, init an
 // op state, call forward / backward, wait on the returned handles and compare.
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <memory>
@@ -75,6 +76,16 @@ PYBIND11_MODULE(_cs_host, m) {
   m.def("clip_grad_norm_", &compute::Utils::clip_grad_norm_, py::arg("scheduler"), py::arg("tensors"),
         py::arg("max_norm"), py::arg("norm_type") = 2.0);
   m.def("from_torch", &memory::from_torch, py::arg("scheduler"), py::arg("tensor"));
+  // what cs::load does with each row of a checkpoint (src/module/module.cpp:216-218): the values,
+  // converted to the parameter's dtype and device and viewed in its shape, are copied into it
+  m.def("assign_", [](const Scheduler &s, const ReadOnlyTensor &parameter, const at::Tensor &values) {
+    parameter.wait();
+    auto &dst = parameter.impl()->tensor();
+    TORCH_CHECK(dst.defined(), "assign_ needs a defined parameter");
+    TORCH_CHECK(values.numel() == dst.numel(), "assign_: ", values.numel(), " values for a parameter of ", dst.numel());
+    (void)dst.copy_(values.to(dst.options()).view(dst.sizes()));
+    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().synchronize();
+  }, py::arg("scheduler"), py::arg("parameter"), py::arg("values"));
 
   py::class_<AutocastScope>(m, "autocast")
       .def(py::init([]() { return AutocastScope{}; }))
