@@ -688,6 +688,12 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
         CS_LN_BWD_MASK(2, CS_LN_BWD_ROWS_VPL2)
       } else if (p.vpl == 4) {
         CS_LN_BWD_MASK(4, CS_LN_BWD_ROWS_VPL4)
+      } else if (dx && want_dp) {
+        // 8 vectors per lane: accumulators, gamma and two rows in flight do not fit in 256
+        // registers together (the single kernel spilled ~1 KB per lane: 225 us at [8192, 4096]
+        // bf16); two passes over dy and x, each within budget, take 85 us
+        CS_LN_BWD(8, 1, true, false, false);
+        CS_LN_BWD(8, 1, false, true, false);
       } else {
         CS_LN_BWD_MASK(8, 1)
       }
