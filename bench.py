@@ -369,6 +369,33 @@ def per_op_table(args, torch, ops):
                     "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
                     "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 3})
         log(f"[per-op] fused_classifier xl          {med*1e3:9.1f} us  {nbytes/med/1e6:8.1f} GB/s")
+        del bufs, x
+        torch.cuda.empty_cache()
+
+    # ---- reference-faithful variants of the headline op, whole call (three launches) each:
+    #      every column a class (V == stride == 50304), and the autocast rule (bf16 logits in,
+    #      fp32 gradient out: test/test_cross_entropy.cpp:102-139)
+    if wanted("fused_classifier"):
+        N = CE_N
+        t = torch.randint(0, CE_V, (N,), generator=g, device=dev, dtype=torch.int64)
+        bufs = [randn((N, CE_STRIDE), 2.0) for _ in range(3)]
+        grads = [torch.empty((N, CE_STRIDE), dtype=torch.float32, device=dev) for _ in range(2)]
+        variants = (
+            ("in place, V 50257", 2 * N * CE_V * 2, lambda i: ops.fused_classifier(bufs[i % 3], t, CE_V, inplace=True)),
+            ("in place, V = stride = 50304", 2 * N * CE_STRIDE * 2,
+             lambda i: ops.fused_classifier(bufs[i % 3], t, CE_STRIDE, inplace=True)),
+            ("bf16 logits -> fp32 gradient (autocast)", N * CE_V * 6,
+             lambda i: ops.fused_classifier(bufs[i % 3], t, CE_V, dlogits_dtype=torch.float32)),
+        )
+        for tag, nbytes, fn in variants:
+            fn(0)
+            med, _ = event_ms(fn, max(5, reps // 4), torch)
+            out.append({"op": "fused_classifier_call", "config": f"[{N},{CE_STRIDE}] bf16, {tag}",
+                        "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
+                        "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
+                        "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 3})
+            log(f"[per-op] fused_classifier call        {tag:42s} {med*1e3:9.1f} us  {nbytes/med/1e6:8.1f} GB/s")
+        del grads
     return out
 
 

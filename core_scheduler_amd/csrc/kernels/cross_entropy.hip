@@ -198,6 +198,27 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
   }
 }
 
+// EPV elements of T in one 8- or 16-byte access.  The streaming kernel reads 16-bit logits 8
+// bytes per lane when it writes fp32 gradients, so that every store is a full 16 bytes per lane
+// and a wave's store covers one contiguous kilobyte (with 16-byte loads each lane would own 32
+// output bytes and every store instruction would touch only half of each 64-byte line).
+template <typename T, int EPV>
+struct alignas(EPV * sizeof(T)) VecE {
+  T e[EPV];
+};
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <typename T, int EPV>
+__device__ __forceinline__ VecE<T, EPV> load_e_stream(const T *p) {
+  static_assert(EPV * sizeof(T) == 16 || EPV * sizeof(T) == 8, "8- or 16-byte accesses");
+  if constexpr (EPV * sizeof(T) == 16) {
+    const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return __builtin_bit_cast(VecE<T, EPV>, raw);
+  } else {
+    const u32x2 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+    return __builtin_bit_cast(VecE<T, EPV>, raw);
+  }
+}
+
 // Streaming variant for wide rows (the GPT-2 vocabulary): one 1024-lane
 // workgroup per CU walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and
 // loads the next row into a second register set before it starts on the
@@ -210,13 +231,13 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
 // e = 2^((x - m_lane) log2e) is kept in registers, one exchange of (max, sum)
 // pairs across the 16 waves gives the row's max and sum, and the output is
 // e * f with one per-lane factor f = 2^(m_lane*log2e - log2(sum) - max*log2e) * s.
-template <typename T, typename TD, int VPT>
+template <typename T, typename TD, int VPT, int EPV>
 __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
     const int *__restrict__ ws_count, int64_t N, int64_t V, int64_t row_stride,
     int64_t ignore_index, int reduction, float dloss) {
   constexpr int BLOCK = 1024;
-  constexpr int VN = Vec16<T>::n;
+  constexpr int VN = EPV;  // elements per lane per access
   constexpr int kWaves = BLOCK / kWave;
   __shared__ float red_m[2][kWaves], red_s[2][kWaves];
   const int tid = threadIdx.x;
@@ -231,7 +252,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   const bool negate = scale < 0.f;
 
   int64_t row = blockIdx.x;
-  Vec16<T> cur[VPT];
+  VecE<T, EPV> cur[VPT];
   int64_t tgt = 0;
   bool live = false;
   float x_t = 0.f;
@@ -243,7 +264,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
 #pragma unroll
       for (int j = 0; j < VPT; ++j) {
         const int idx = tid + BLOCK * j;
-        if (idx < nvec) cur[j] = load16_stream(x + (int64_t)idx * VN);
+        if (idx < nvec) cur[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
       }
       if (tid == 0) x_t = to_acc(x[tgt]);
     }
@@ -252,7 +273,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   while (row < N) {
     // ---- issue the next row's loads
     const int64_t nrow = row + gridDim.x;
-    Vec16<T> nxt[VPT];
+    VecE<T, EPV> nxt[VPT];
     int64_t ntgt = 0;
     bool nlive = false;
     float nx_t = 0.f;
@@ -264,7 +285,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
           const int idx = tid + BLOCK * j;
-          if (idx < nvec) nxt[j] = load16_stream(x + (int64_t)idx * VN);
+          if (idx < nvec) nxt[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
         }
         if (tid == 0) nx_t = to_acc(x[ntgt]);
       }
@@ -441,15 +462,23 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         // one persistent workgroup per CU
         const int64_t cus = compute_units();
         const dim3 pgrid((unsigned)(N < cus ? N : cus));
-        if (nvec <= 1024 * 7) {
-          ce_rows_stream_kernel<T, TD, 7><<<pgrid, dim3(1024), 0, s>>>(
-              (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,
-              ignore_index, reduction, dloss);
+#define CS_CE_STREAM(VPT, EPV)                                                              \
+  ce_rows_stream_kernel<T, TD, VPT, EPV><<<pgrid, dim3(1024), 0, s>>>(                      \
+      (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,      \
+      ignore_index, reduction, dloss)
+        if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
+          // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
+          if (nvec * 2 <= 1024 * 13) {
+            CS_CE_STREAM(13, 4);
+          } else {
+            CS_CE_STREAM(16, 4);
+          }
+        } else if (nvec <= 1024 * 7) {
+          CS_CE_STREAM(7, VN);
         } else {
-          ce_rows_stream_kernel<T, TD, 8><<<pgrid, dim3(1024), 0, s>>>(
-              (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,
-              ignore_index, reduction, dloss);
+          CS_CE_STREAM(8, VN);
         }
+#undef CS_CE_STREAM
       } else {
         CS_CE(1024, 16);
       }

@@ -564,6 +564,23 @@ def test_cross_entropy_inplace_amp_and_dloss(ops, co):
     assert none is None and loss3.item() == loss.item()
 
 
+@pytest.mark.parametrize("N,V,stride", [(300, 50257, 50304), (270, 59990, 60000), (5, 65536, 65536)])
+def test_cross_entropy_autocast_wide_rows(ops, co, N, V, stride):
+    """16-bit logits with fp32 gradients on the streaming kernel's two register plans, with more
+    rows than workgroups (so rows are prefetched) and ignored rows among them."""
+    x = randn((N, stride), 116, std=2.0, dtype=torch.bfloat16)
+    t = randint(0, V, (N,), 117)
+    t[1] = -100
+    t[N - 1] = -100
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t), V, dlogits_dtype=torch.float32)
+    loss2, row2, d2, tw2 = co.cross_entropy(x, t, V, dlogits_dtype=torch.float32)
+    assert d.dtype == torch.float32 and tw.item() == tw2.item() == N - 2
+    assert_close(loss, loss2.float(), atol=1e-5, name="loss")
+    assert_close(row, row2.float(), atol=1e-5, name="row loss")
+    assert_close(d, d2, atol=1e-10, name="dlogits")
+    assert (d[:, V:] == 0).all() and (d[1] == 0).all()
+
+
 def test_cross_entropy_all_ignored_and_bad_targets(ops):
     x = randn((6, 128), 115, dtype=torch.bfloat16)
     t = torch.full((6,), -100, dtype=torch.int64)
