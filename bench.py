@@ -502,7 +502,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "ce_rows_kernel<bf16, bf16, 1024, 7>",
+            "kernel": "ce_rows_stream_kernel<bf16_t, bf16_t, 7, 8>",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
