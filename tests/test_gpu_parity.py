@@ -695,3 +695,43 @@ def test_xl_adamw(ops, co):
     assert (m_all != 0).all()
     del opt, w, grad
     torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------- empty inputs
+def test_empty_inputs(ops, co):
+    """Zero rows / tokens / elements: every call returns without launching anything harmful and
+    leaves well-defined outputs (an embedding gradient for no tokens is all zeros)."""
+    z = torch.empty((0, 768), dtype=torch.bfloat16, device=DEV)
+    gamma, beta = torch.ones(768, device=DEV), torch.zeros(768, device=DEV)
+    y, mean, rstd = ops.layernorm_forward(z, gamma, beta)
+    assert y.shape == (0, 768) and mean.numel() == 0
+    dx, dg, db = ops.layernorm_backward(z, z, mean, rstd, gamma)
+    assert dx.shape == (0, 768)
+    assert ops.gelu_forward(z).shape == (0, 768) and ops.gelu_backward(z, z).shape == (0, 768)
+    # embedding: no tokens -> an empty activation, a zero gradient (and an untouched one when accumulating)
+    wte = randn((50, 16), 1, dtype=torch.bfloat16)
+    ids = torch.empty((0, 8), dtype=torch.int64, device=DEV)
+    assert ops.embedding_forward(dev(wte), ids).shape == (0, 8, 16)
+    dw = ops.embedding_backward(torch.empty((0, 8, 16), dtype=torch.bfloat16, device=DEV), ids, 50)
+    assert dw.shape == (50, 16) and (dw == 0).all()
+    keep = dev(wte).clone()
+    ops.embedding_backward(torch.empty((0, 8, 16), dtype=torch.bfloat16, device=DEV), ids, 50, dweight=keep)
+    assert_bit_exact(keep, wte, "accumulating nothing")
+    # AdamW: an empty tensor alone, and one among others in the multi-tensor table
+    e = torch.empty(0, device=DEV)
+    ops.adamw_step(e, e, e, e, t=1, **HYPER)
+    ws = [randn((5,), 2), torch.empty(0), randn((4097,), 3)]
+    gs = [randn((5,), 4), torch.empty(0), randn((4097,), 5)]
+    gws = [dev(w) for w in ws]
+    opt = ops.MultiTensorAdamW(gws, [dev(g) for g in gs], t=0, **HYPER)
+    opt.step()
+    for i in (0, 2):
+        w2, _, _, _ = co.adamw_step(ws[i], gs[i], torch.zeros_like(ws[i]), torch.zeros_like(ws[i]), t=1, **HYPER)
+        assert_close(gws[i], w2, atol=1e-8, name=f"w[{i}]")
+    # cross entropy over no rows: sum is 0, mean is 0/0
+    x = torch.empty((0, 128), dtype=torch.bfloat16, device=DEV)
+    t = torch.empty((0,), dtype=torch.int64, device=DEV)
+    loss, row, d, tw = ops.fused_classifier(x, t, 100, reduction="sum")
+    assert loss.item() == 0 and tw.item() == 0 and d.shape == (0, 128)
+    loss, _, _, _ = ops.fused_classifier(x, t, 100)
+    assert math.isnan(loss.item())
