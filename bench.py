@@ -425,6 +425,56 @@ def cpu_baseline(args, torch):
     }
 
 
+def cpu_per_op(args, torch, table):
+    """The reference's CPU path for every small-configuration row of the per-op table: the ATen
+    CPU ops its task bodies call (fp32 inputs, as its CPU tests run them) and, for AdamW, the C
+    restatement of its kernel.  Attaches `cpu_ms` (median of 3 after a warm-up) to the records."""
+    from oracle import aten_port as ap
+    from oracle import c_oracle as co
+
+    g = torch.Generator().manual_seed(1337)
+
+    def med(fn, reps=3):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts) * 1e3
+
+    cpu = {}
+    rows, C = 8192, 768
+    x, dy = torch.randn((rows, C), generator=g), torch.randn((rows, C), generator=g)
+    gamma, beta = torch.ones(C), torch.zeros(C)
+    _, mean, rstd = ap.layernorm_forward(x, gamma, beta)
+    cpu[("layernorm_fwd", "small")] = med(lambda: ap.layernorm_forward(x, gamma, beta))
+    cpu[("layernorm_bwd", "small")] = med(lambda: ap.layernorm_backward(dy, x, mean, rstd, gamma, beta))
+    xg, dg = torch.randn(8192 * 3072, generator=g) * 1.5, torch.randn(8192 * 3072, generator=g)
+    for mode, tag in (("tanh", "tanh"), ("none", "erf")):
+        cpu[(f"gelu_fwd_{tag}", "")] = med(lambda: ap.gelu_forward(xg, mode))
+        cpu[(f"gelu_bwd_{tag}", "")] = med(lambda: ap.gelu_backward(dg, xg, mode))
+    V, B, T = 50257, 8, 1024
+    wte, wpe = torch.randn((V, C), generator=g) * 0.02, torch.randn((T, C), generator=g) * 0.02
+    ids = torch.randint(0, V, (B, T), generator=g)
+    dout = torch.randn((B, T, C), generator=g)
+    cpu[("embedding_fwd", "small uniform")] = med(lambda: ap.token_position_forward(wte, wpe, ids))
+    cpu[("embedding_bwd", "small uniform")] = med(lambda: ap.token_position_backward(dout, ids, V))
+    total = sum(gpt2_param_sizes(12, 768))
+    w, gr = torch.randn(total, generator=g) * 0.02, torch.randn(total, generator=g) * 1e-3
+    m, v = torch.zeros(total), torch.zeros(total)
+    hp = dict(lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    cpu[("adamw_multi_tensor", "small")] = med(lambda: co.adamw_step(w, gr, m, v, t=1, **hp), reps=2)
+    for rec in table:
+        for (op, tag), ms in cpu.items():
+            if rec["op"] == op and rec["config"].startswith(tag):
+                rec["cpu_ms"] = round(ms, 3)
+                rec["cpu_path"] = ("C restatement of src/optimizer/adamw.cu, 1 thread" if op.startswith("adamw")
+                                   else f"ATen CPU ops of the reference's task body, fp32, {torch.get_num_threads()} threads")
+                log(f"[cpu]    {op:28s} {rec['config'][:34]:34s} {ms:10.2f} ms on the CPU, {rec['ms_cold']*1e3:9.1f} us on the GPU")
+    return table
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -479,6 +529,8 @@ def main():
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(args, torch)
         log(f"[bench] CPU baseline (ATen CPU, {cpu['cores']} threads): {cpu['ms']:.1f} ms, {cpu['value']} GB/s")
+        if table:
+            cpu_per_op(args, torch, table)
 
     line = {
         "metric": "fused CE HBM GB/s at 8192x50257 bf16 (ms in ms_per_step; every op in per_op)",

@@ -609,7 +609,10 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
 // Grid caps: beyond these the waves loop over rows (with prefetch) instead of
 // the grid growing, which keeps the parameters in registers for many rows
 // and bounds the number of partial rows the backward pass leaves behind.
-constexpr int kLnFwdMaxBlocks = 1024;
+#ifndef CS_LN_FWD_MAX_BLOCKS
+#define CS_LN_FWD_MAX_BLOCKS 1024
+#endif
+constexpr int kLnFwdMaxBlocks = CS_LN_FWD_MAX_BLOCKS;
 constexpr int kLnBwdMaxBlocks = CS_LN_BWD_MAX_BLOCKS;
 
 int ln_blocks(int64_t rows, int rows_per_wave, int cap, int threads = kLnThreads) {
