@@ -375,6 +375,165 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
   }
 }
 
+// ------------------------------------------------- wide rows: two waves per row
+// Rows of 5 to 8 vectors per lane do not fit one wave's registers once the dgamma/dbeta
+// accumulators are there, so a pair of waves shares a row: wave h of the pair (h = 0, 1) owns
+// vectors lane + 64*(2j + h), j < VPLH.  The two halves of the row sums meet in the LDS (one
+// barrier per row; every pair makes the same number of steps so that all waves reach it).
+template <typename T, int VN, int VPLH>
+struct HalfRow {
+  Raw<T, VN> v[VPLH];
+};
+template <typename T, int VN, int VPLH>
+__device__ __forceinline__ void load_half_row(HalfRow<T, VN, VPLH> &dst, const T *__restrict__ src,
+                                              int64_t row, bool valid, int C, int nvec, int lane, int h) {
+#pragma unroll
+  for (int j = 0; j < VPLH; ++j) {
+    const int idx = lane + kWave * (2 * j + h);
+    if (valid && idx < nvec) {
+      dst.v[j] = load_raw<T, VN>(src + row * C + (int64_t)idx * VN);
+    } else {
+      dst.v[j] = zero_raw<T, VN>();
+    }
+  }
+}
+
+template <typename TDY, typename TX, typename TDX, typename TP, int VPLH, bool HAS_DX, bool HAS_DP>
+__global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_split_rows_kernel(
+    const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
+    const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
+    float *__restrict__ partial, int64_t rows, int C) {
+  constexpr int VN = Vec16<TX>::n;
+  constexpr int kWaves = kLnBwdThreads / kWave;
+  constexpr int kPairs = kWaves / 2;
+  constexpr int kRegion = VPLH * kWave * VN;  // floats one wave contributes to the fold
+  extern __shared__ float lds[];              // [kPairs][kRegion], one half of the row at a time
+  __shared__ float halves[2][kPairs][2][2];   // [parity][pair][half][s1, s2]
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int pair = wave >> 1, h = wave & 1;
+  const int64_t n_pairs = (int64_t)gridDim.x * kPairs;
+  const int64_t gp = (int64_t)blockIdx.x * kPairs + pair;
+  const int64_t steps = (rows + n_pairs - 1) / n_pairs;  // the same for every pair
+  const int nvec = C / VN;
+  const float inv_c = 1.0f / (float)C;
+
+  float acc_g[VPLH][VN], acc_b[VPLH][VN], g[VPLH][VN];
+#pragma unroll
+  for (int j = 0; j < VPLH; ++j) {
+    const int idx = lane + kWave * (2 * j + h);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      acc_g[j][k] = 0.f;
+      acc_b[j][k] = 0.f;
+      g[j][k] = 0.f;
+    }
+    if (HAS_DX && idx < nvec) load_n<TP, VN>(gamma + idx * VN, g[j]);
+  }
+
+  HalfRow<TDY, VN, VPLH> dcur;
+  HalfRow<TX, VN, VPLH> xcur;
+  int64_t row = gp;
+  load_half_row<TDY, VN, VPLH>(dcur, dy, row, row < rows, C, nvec, lane, h);
+  load_half_row<TX, VN, VPLH>(xcur, x, row, row < rows, C, nvec, lane, h);
+  float mu = row < rows ? mean[row] : 0.f, rs = row < rows ? rstd[row] : 0.f;
+  int parity = 0;
+  for (int64_t it = 0; it < steps; ++it, row += n_pairs) {
+    const int64_t nrow = row + n_pairs;
+    HalfRow<TDY, VN, VPLH> dnxt;
+    HalfRow<TX, VN, VPLH> xnxt;
+    load_half_row<TDY, VN, VPLH>(dnxt, dy, nrow, nrow < rows, C, nvec, lane, h);
+    load_half_row<TX, VN, VPLH>(xnxt, x, nrow, nrow < rows, C, nvec, lane, h);
+    const float nmu = nrow < rows ? mean[nrow] : 0.f, nrs = nrow < rows ? rstd[nrow] : 0.f;
+
+    // a row past the end is all zeros here: it adds nothing and stores nothing
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPLH; ++j) {
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        const float xh = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
+        const float dv = raw_get<TDY, VN>(dcur.v[j], k);
+        if constexpr (HAS_DP) {
+          acc_g[j][k] += dv * xh;
+          acc_b[j][k] += dv;
+        }
+        if constexpr (HAS_DX) {
+          const float gd = dv * g[j][k];
+          s1 += gd;
+          s2 += gd * xh;
+        }
+      }
+    }
+    if constexpr (HAS_DX) {
+      s1 = wave_reduce(s1, SumOp{});
+      s2 = wave_reduce(s2, SumOp{});
+      if (lane == 0) {
+        halves[parity][pair][h][0] = s1;
+        halves[parity][pair][h][1] = s2;
+      }
+      __syncthreads();
+      // both waves of the pair add the halves in the same order
+      s1 = (halves[parity][pair][0][0] + halves[parity][pair][1][0]) * inv_c;
+      s2 = (halves[parity][pair][0][1] + halves[parity][pair][1][1]) * inv_c;
+      parity ^= 1;  // the other buffer next step: one barrier per row is enough
+      if (row < rows) {
+#pragma unroll
+        for (int j = 0; j < VPLH; ++j) {
+          forget_unpacked(xcur.v[j]);
+          forget_unpacked(dcur.v[j]);
+          const int idx = lane + kWave * (2 * j + h);
+          if (idx < nvec) {
+            float o[VN];
+#pragma unroll
+            for (int k = 0; k < VN; ++k) {
+              const float xh = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
+              const float dv = raw_get<TDY, VN>(dcur.v[j], k);
+              o[k] = rs * (dv * g[j][k] - s1 - xh * s2);
+            }
+            store_n<TDX, VN>(dx + row * C + (int64_t)idx * VN, o);
+          }
+        }
+      }
+    }
+    dcur = dnxt;
+    xcur = xnxt;
+    mu = nmu;
+    rs = nrs;
+  }
+
+  if constexpr (HAS_DP) {
+    // fold the four waves that own the same half, one half at a time; positions inside a wave's
+    // region are k*(64 VPLH) + lane + 64 j (conflict-free writes); the partial rows use the
+    // permuted layout of the narrow kernel, position k*nvec + idx for column idx*VN + k
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        if (h == hh) {
+#pragma unroll
+          for (int j = 0; j < VPLH; ++j)
+#pragma unroll
+            for (int k = 0; k < VN; ++k)
+              lds[pair * kRegion + k * (kWave * VPLH) + lane + kWave * j] = which == 0 ? acc_g[j][k] : acc_b[j][k];
+        }
+        __syncthreads();
+        for (int local = threadIdx.x; local < kRegion; local += kLnBwdThreads) {
+          const int k = local / (kWave * VPLH), li = local % (kWave * VPLH);
+          const int idx = (li % kWave) + kWave * (2 * (li / kWave) + hh);
+          if (idx < nvec) {
+            float sum = 0.f;
+#pragma unroll
+            for (int pp = 0; pp < kPairs; ++pp) sum += lds[pp * kRegion + local];
+            partial[((int64_t)blockIdx.x * 2 + which) * C + k * nvec + idx] = sum;
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+}
+
 // Adds `nparts` partial rows in a fixed order.  Partial rows are permuted: position
 // p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  grid (ceil(C/64), 2), block
 // (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one column
@@ -666,7 +825,10 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
       const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks, kLnBwdThreads);
-      const size_t need = want_dp ? (size_t)blocks * 2 * C * sizeof(float) : 0;
+      // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
+      const int split_blocks = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
+      int blocks_used = p.vpl == 8 && want_dp ? split_blocks : blocks;  // partial rows left behind
+      const size_t need = want_dp ? (size_t)blocks_used * 2 * C * sizeof(float) : 0;
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
       const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
       const dim3 grid((unsigned)blocks), block(kLnBwdThreads);
@@ -691,21 +853,29 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
         CS_LN_BWD_MASK(2, CS_LN_BWD_ROWS_VPL2)
       } else if (p.vpl == 4) {
         CS_LN_BWD_MASK(4, CS_LN_BWD_ROWS_VPL4)
-      } else if (dx && want_dp) {
-        // 8 vectors per lane: accumulators, gamma and two rows in flight do not fit in 256
-        // registers together (the single kernel spilled ~1 KB per lane: 225 us at [8192, 4096]
-        // bf16); two passes over dy and x, each within budget, take 85 us
-        CS_LN_BWD(8, 1, true, false, false);
-        CS_LN_BWD(8, 1, false, true, false);
+      } else if (want_dp) {
+        // 8 vectors per lane: with the dgamma/dbeta accumulators a row no longer fits one wave's
+        // registers (a single-wave kernel spilled ~1 KB per lane), so two waves share each row
+        const size_t split_lds = (size_t)(kLnBwdThreads / kWave / 2) * 4 * kWave * Vec16<TX>::n * sizeof(float);
+        const dim3 sgrid((unsigned)split_blocks);
+        if (dx) {
+          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, true, true><<<sgrid, block, split_lds, s>>>(
+              (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd, (const TP *)gamma,
+              (TDX *)dx, (float *)workspace, rows, (int)C);
+        } else {
+          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, false, true><<<sgrid, block, split_lds, s>>>(
+              (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd, (const TP *)gamma,
+              (TDX *)dx, (float *)workspace, rows, (int)C);
+        }
       } else {
-        CS_LN_BWD_MASK(8, 1)
+        CS_LN_BWD(8, 1, true, false, false);
       }
 #undef CS_LN_BWD_MASK
 #undef CS_LN_BWD
       int st = launch_status();
       if (st == CS_OK && want_dp) {
         ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
-            (const float *)workspace, blocks, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
+            (const float *)workspace, blocks_used, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
         st = launch_status();
       }
       if (st == CS_OK && late_dres) st = launch_add<TDX>(dx, late_dres, dx, rows * C, s);
@@ -808,8 +978,8 @@ extern "C" int cs_add_layernorm_forward(const void *x, const void *residual, voi
 
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
-  // the fast path's largest grid: one row per wave per step
-  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads) * 2 * (size_t)C * sizeof(float);
+  // the fast path's largest grid: one row per pair of waves per step
+  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2) * 2 * (size_t)C * sizeof(float);
 }
 
 namespace {

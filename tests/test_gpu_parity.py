@@ -279,7 +279,10 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
     (1024, 384, torch.float32, torch.float32),      # test/test_layer_norm.cpp:63-96 width
     (513, 768, torch.float16, torch.float16),
     (300, 768, torch.bfloat16, torch.bfloat16),
-    (77, 4096, torch.bfloat16, torch.float32),      # 8 vectors per lane plan
+    (77, 4096, torch.bfloat16, torch.float32),      # 8 vectors per lane plan: two waves per row backward
+    (2051, 1600, torch.float32, torch.float32),     # the same plan from fp32 rows, rows not a multiple of anything
+    (3, 4096, torch.float16, torch.float16),        # fewer rows than wave pairs
+    (1100, 2056, torch.bfloat16, torch.float32),    # just over 4 vectors per lane, several rows per pair
     (5, 768, torch.float32, torch.float32),         # fewer rows than one workgroup
     (64, 50, torch.float32, torch.float32),         # C not a multiple of the vector width
     (33, 10000, torch.bfloat16, torch.float32),     # beyond the register plans
