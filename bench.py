@@ -533,7 +533,8 @@ def main():
             cpu_per_op(args, torch, table)
 
     line = {
-        "metric": "fused CE HBM GB/s at 8192x50257 bf16 (ms in ms_per_step; every op in per_op)",
+        "metric": "per-op HBM GB/s (% of MI355X peak); fused CE ms at 8192x50257 bf16",
+        "metric_note": "value = the fused classifier's whole-step GB/s (the ms is ms_per_step); every other op is in per_op",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
