@@ -490,6 +490,44 @@ def test_embedding_backward_padding_accumulate_and_bad_ids(ops, co):
                  name="out-of-range ids are skipped")
 
 
+def test_embedding_backward_random_cases(ops, co):
+    """Seeded random shapes around the kernel's internal boundaries (32-entry windows, 4-entry
+    waves, 1024-key tiles, the 32/64-bit key switch) with id patterns that stress each level of
+    the segmented sum: one hot id, a sorted stream, a single id, a padding row; `=` and `+=`."""
+    import random
+
+    rnd = random.Random(7)
+    for case in range(80):
+        n = rnd.choice([1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 1000, 1023, 1024, 1025, 2047, 2049, 3000, 5000, 9000])
+        V = rnd.choice([1, 2, 3, 7, 33, 100, 1000, 5000, 70000])
+        C = rnd.choice([8, 16, 64, 200, 768, 1032])
+        dt = rnd.choice([torch.bfloat16, torch.float32, torch.float16])
+        kind = rnd.choice(["uniform", "hot", "sorted", "allsame", "padding"])
+        g = torch.Generator().manual_seed(case)
+        ids = torch.randint(0, V, (n,), generator=g)
+        if kind == "hot":
+            ids = torch.where(torch.rand(n, generator=g) < 0.7, torch.full((n,), V // 2), ids)
+        elif kind == "sorted":
+            ids = torch.sort(ids)[0]
+        elif kind == "allsame":
+            ids = torch.full((n,), V - 1, dtype=torch.int64)
+        kw = dict(padding_idx=V // 3) if kind == "padding" else {}
+        if rnd.random() < 0.3:
+            ids = ids.to(torch.int32)
+        dout = torch.randn((n, C), generator=g).to(dt)
+        tag = f"case {case}: n={n} V={V} C={C} {dt} {kind}"
+        if rnd.random() < 0.3:
+            base = torch.randn((V, C), generator=g).to(dt)
+            got = dev(base).clone()
+            ops.embedding_backward(dev(dout), dev(ids), V, dweight=got, **kw)
+            want = co.embedding_backward(dout, ids, V, dweight=base, **kw)
+        else:
+            got = ops.embedding_backward(dev(dout), dev(ids), V, **kw)
+            want = co.embedding_backward(dout, ids, V, **kw)
+        # sums of up to n N(0,1) terms in fp32: a few e-5 absolute at n = 9000
+        assert_close(got, want, atol=2e-4, name=tag)
+
+
 @pytest.mark.parametrize("kind", ["uniform", "zipf"])
 def test_embedding_config1(ops, co, kind):
     """Benchmark configuration 1: wte 50257x768, wpe 1024x768 bf16, B 8, T 1024."""
