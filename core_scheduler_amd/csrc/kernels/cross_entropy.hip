@@ -147,26 +147,29 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
     const int c0 = (tid + BLOCK * j) * VN;
     if (c0 + VN <= iV) {
 #pragma unroll
-      for (int k = 0; k < VN; ++k) s += __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - m2);
+      for (int k = 0; k < VN; ++k) s += __builtin_amdgcn_exp2f(__builtin_fmaf(vec_get(xr[j], k), kLog2e, -m2));
     } else if (c0 < iV) {
 #pragma unroll
       for (int k = 0; k < VN; ++k)
-        if (c0 + k < iV) s += __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - m2);
+        if (c0 + k < iV) s += __builtin_amdgcn_exp2f(__builtin_fmaf(vec_get(xr[j], k), kLog2e, -m2));
     }
   }
   s = block_reduce(s, SumOp{}, 0.f, scratch);
 
   const float log2_s = __builtin_amdgcn_logf(s);  // v_log_f32 is log2
-  if (tid == 0 && row_loss) row_loss[row] = (m2 + log2_s) * kLn2 - x_t;
+  // loss = ln(sum exp(x - max)) - (x_t - max): the difference to the maximum is formed with one
+  // fused multiply-add against the same rounded m2 the sum used, so a loss near 0 keeps its digits
+  if (tid == 0 && row_loss) row_loss[row] = (log2_s - __builtin_fmaf(x_t, kLog2e, -m2)) * kLn2;
   if (dlogits == nullptr) return;
 
-  // ---- dlogits = (p - onehot) * scale, p * scale = 2^(x*log2e - K)
+  // ---- dlogits = (p - onehot) * scale with p = 2^(x*log2e - m2) / s.  The exponent is taken
+  // relative to the row maximum with one fused multiply-add, the same expression the sum above
+  // used, so the rounding of m2 cancels between numerator and denominator and p keeps fp32
+  // accuracy; folding log2(s) and log2(scale) into the exponent instead costs ~1e-6 relative,
+  // which the subtraction at the target column amplifies when p is close to 1.
   float scale = dloss;
   if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
-  // K folds max, sum and |scale|; the sign of scale is applied afterwards
-  const float abs_scale = fabsf(scale);
-  const float K = m2 + log2_s - __builtin_amdgcn_logf(abs_scale);
-  const float sign = scale < 0.f ? -1.f : 1.f;
+  const float factor = scale / s;  // s >= 1: the maximum contributes 2^0
   const int t_vec = (int)(target / VN), t_sub = (int)(target % VN);
   TD *d = dlogits + row * row_stride;
 #pragma unroll
@@ -175,14 +178,9 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
     if (idx < nvec) {
       const int c0 = idx * VN;
       float o[VN];
-      if (abs_scale == 0.f) {
 #pragma unroll
-        for (int k = 0; k < VN; ++k) o[k] = 0.f;
-      } else {
-#pragma unroll
-        for (int k = 0; k < VN; ++k)
-          o[k] = sign * __builtin_amdgcn_exp2f(vec_get(xr[j], k) * kLog2e - K);
-      }
+      for (int k = 0; k < VN; ++k)
+        o[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(vec_get(xr[j], k), kLog2e, -m2)) * factor;
       if (c0 + VN > iV) {  // last class vector and the padding
 #pragma unroll
         for (int k = 0; k < VN; ++k)
@@ -230,7 +228,7 @@ __device__ __forceinline__ VecE<T, EPV> load_e_stream(const T *p) {
 // Each element costs one hardware exp2: lane-local max first, then
 // e = 2^((x - m_lane) log2e) is kept in registers, one exchange of (max, sum)
 // pairs across the 16 waves gives the row's max and sum, and the output is
-// e * f with one per-lane factor f = 2^(m_lane*log2e - log2(sum) - max*log2e) * s.
+// e * f with one per-lane factor f = 2^(m_lane*log2e - log2(sum) - max*log2e) * scale.
 template <typename T, typename TD, int VPT, int EPV>
 __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
@@ -255,7 +253,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   VecE<T, EPV> cur[VPT];
   int64_t tgt = 0;
   bool live = false;
-  float x_t = 0.f;
   if (row < N) {
     tgt = targets[row];
     live = target_counts(tgt, V, ignore_index);
@@ -266,7 +263,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
         const int idx = tid + BLOCK * j;
         if (idx < nvec) cur[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
       }
-      if (tid == 0) x_t = to_acc(x[tgt]);
     }
   }
   int parity = 0;
@@ -276,7 +272,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     VecE<T, EPV> nxt[VPT];
     int64_t ntgt = 0;
     bool nlive = false;
-    float nx_t = 0.f;
     if (nrow < N) {
       ntgt = targets[nrow];
       nlive = target_counts(ntgt, V, ignore_index);
@@ -287,7 +282,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
           const int idx = tid + BLOCK * j;
           if (idx < nvec) nxt[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
         }
-        if (tid == 0) nx_t = to_acc(x[ntgt]);
       }
     }
 
@@ -301,6 +295,12 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
           store_out<T, TD, VN>(dlogits + row * row_stride + (int64_t)idx * VN, z);
       }
     } else {
+      // the target column sits in vector t_vec = j_t * BLOCK + tid_t, element t_sub: a uniform
+      // test on j and a per-lane element index keep its handling out of the other vectors
+      const int t_vec = (int)(tgt / VN);
+      const int j_t = t_vec / BLOCK;
+      const int my_sub = (t_vec % BLOCK) == tid ? (int)(tgt % VN) : -1;
+      float x_t = 0.f;  // the target's logit, in the lane that holds it
       // ---- widen, mask what is not a class column to -inf, lane-local max
       float e[VPT][VN];
       float m = -INFINITY;
@@ -319,6 +319,10 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
             e[j][k] = c0 + k < iV ? to_acc(cur[j].e[k]) : -INFINITY;
             m = fmaxf(m, e[j][k]);
           }
+        }
+        if (j == j_t) {  // uniform
+#pragma unroll
+          for (int k = 0; k < VN; ++k) x_t = k == my_sub ? e[j][k] : x_t;
         }
       }
       // a lane without any class column: any finite stand-in keeps 2^(-inf - m) = 0
@@ -345,14 +349,19 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
       const float S = wave_reduce(ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
       parity ^= 1;  // the other pair of arrays next time: one barrier per row is enough
       const float log2_S = __builtin_amdgcn_logf(S);
-      if (tid == 0 && row_loss) row_loss[row] = (M2 + log2_S) * kLn2 - x_t;
+      // loss = ln(sum exp(x - max)) - (x_t - max), the difference to the maximum formed with one
+      // fused multiply-add against the rounded M2 the sum was taken with
+      if (my_sub >= 0 && row_loss) row_loss[row] = (log2_S - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
 
       if (dlogits) {
         // a lane that holds no class column has e = 0 everywhere; give it f = 0 so that
         // 0 * f cannot meet an overflowed factor
+        // One factor per lane folds the step from the lane's maximum to the row's, 1/sum and
+        // |scale| into a single exponent.  The logarithms in it are good to ~1e-6 relative,
+        // which is fine everywhere except at the target column, where subtracting `scale`
+        // amplifies it when p is close to 1: that one element is formed as a product instead.
         float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml2 - M2 - log2_S + log2_scale);
         f = negate ? -f : f;
-        const int t_vec = (int)(tgt / VN), t_sub = (int)(tgt % VN);
         TD *d = dlogits + row * row_stride;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
@@ -361,10 +370,10 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
             float o[VN];
 #pragma unroll
             for (int k = 0; k < VN; ++k) o[k] = e[j][k] * f;
-            if (idx == t_vec) {
+            if (j == j_t) {  // uniform
+              const float exact = __builtin_amdgcn_exp2f(ml2 - M2) * (scale * __builtin_amdgcn_rcpf(S));
 #pragma unroll
-              for (int k = 0; k < VN; ++k)
-                if (k == t_sub) o[k] -= scale;
+              for (int k = 0; k < VN; ++k) o[k] = k == my_sub ? e[j][k] * exact - scale : o[k];
             }
             store_out<T, TD, VN>(d + (int64_t)idx * VN, o);
           }
@@ -375,7 +384,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     for (int j = 0; j < VPT; ++j) cur[j] = nxt[j];
     live = nlive;
     tgt = ntgt;
-    x_t = nx_t;
     row = nrow;
   }
 }

@@ -693,7 +693,9 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_dx_general_kernel(
   }
 }
 
-// grid ceil(C/64) blocks of (64, 4): thread (cx, ry) walks rows ry, ry+4, ...
+// grid ceil(C/64) blocks of (64, 4): thread (cx, ry) walks rows ry, ry+4, ...  A thread adds
+// rows/4 terms one after the other, so the running sums are kept in double: in float the
+// rounding of a sum of thousands of O(1) terms reaches several 1e-5.
 template <typename TDY, typename TX, typename TP>
 __global__ __launch_bounds__(256) void ln_bwd_param_general_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x,
@@ -701,32 +703,32 @@ __global__ __launch_bounds__(256) void ln_bwd_param_general_kernel(
     const typename Acc<TX>::type *__restrict__ rstd, TP *__restrict__ dgamma,
     TP *__restrict__ dbeta, int64_t rows, int64_t C, int accumulate) {
   using U = typename Acc<TX>::type;
-  __shared__ U sg[4][64], sb[4][64];
+  __shared__ double sg[4][64], sb[4][64];
   const int64_t col = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  U ag = 0, ab = 0;
+  double ag = 0, ab = 0;
   if (col < C) {
     for (int64_t r = threadIdx.y; r < rows; r += 4) {
       const U d = to_acc(dy[r * C + col]);
-      ag += d * (((U)to_acc(x[r * C + col]) - mean[r]) * rstd[r]);
-      ab += d;
+      ag += (double)(d * (((U)to_acc(x[r * C + col]) - mean[r]) * rstd[r]));
+      ab += (double)d;
     }
   }
   sg[threadIdx.y][threadIdx.x] = ag;
   sb[threadIdx.y][threadIdx.x] = ab;
   __syncthreads();
   if (threadIdx.y == 0 && col < C) {
-    U tg = 0, tb = 0;
+    double tg = 0, tb = 0;
     for (int r = 0; r < 4; ++r) {
       tg += sg[r][threadIdx.x];
       tb += sb[r][threadIdx.x];
     }
     if (dgamma) {
-      if (accumulate) tg += (U)to_acc(dgamma[col]);
-      dgamma[col] = from_acc<TP>(tg);
+      if (accumulate) tg += (double)to_acc(dgamma[col]);
+      dgamma[col] = from_acc<TP>((typename Acc<TP>::type)tg);
     }
     if (dbeta) {
-      if (accumulate) tb += (U)to_acc(dbeta[col]);
-      dbeta[col] = from_acc<TP>(tb);
+      if (accumulate) tb += (double)to_acc(dbeta[col]);
+      dbeta[col] = from_acc<TP>((typename Acc<TP>::type)tb);
     }
   }
 }

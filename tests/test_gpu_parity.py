@@ -285,6 +285,7 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
     (1100, 2056, torch.bfloat16, torch.float32),    # just over 4 vectors per lane, several rows per pair
     (5, 768, torch.float32, torch.float32),         # fewer rows than one workgroup
     (64, 50, torch.float32, torch.float32),         # C not a multiple of the vector width
+    (2049, 50, torch.float32, torch.float32),       # the same with long column sums
     (33, 10000, torch.bfloat16, torch.float32),     # beyond the register plans
     (128, 384, torch.float64, torch.float64),       # test/test_layer_norm.cpp:99-134
 ])
@@ -620,6 +621,35 @@ def test_cross_entropy_autocast_wide_rows(ops, co, N, V, stride):
     assert_close(row, row2.float(), atol=1e-5, name="row loss")
     assert_close(d, d2, atol=1e-10, name="dlogits")
     assert (d[:, V:] == 0).all() and (d[1] == 0).all()
+
+
+@pytest.mark.parametrize("N,V,stride,dtype,gdt", [(600, 17, 64, torch.bfloat16, torch.float32),
+                                                   (64, 1000, 1024, torch.float32, None),
+                                                   (300, 50257, 50304, torch.bfloat16, None),
+                                                   (300, 50257, 50304, torch.bfloat16, torch.float32),
+                                                   (16, 100000, 100000, torch.bfloat16, None)])
+def test_cross_entropy_confident_predictions(ops, co, N, V, stride, dtype, gdt):
+    """Targets the model is nearly sure of: p close to 1 makes (p - 1) a cancellation, so a
+    relative error of 1e-6 in p (what folding the normalisation into one exponent costs) would
+    show as 1e-5 .. 1e-4 in the gradient at the target column."""
+    x = randn((N, stride), 118, std=2.0, dtype=dtype)
+    t = randint(0, V, (N,), 119)
+    boost = torch.linspace(8.0, 20.0, N)  # p_target from ~0.9 to 1 - 1e-6
+    x[torch.arange(N), t] = (x[torch.arange(N), t].float() + boost).to(dtype)
+    kw = dict(dlogits_dtype=gdt) if gdt else {}
+    loss, row, d, _ = ops.fused_classifier(dev(x), dev(t), V, **kw)
+    loss2, row2, d2, _ = co.cross_entropy(x, t, V, **kw)
+    assert_close(row, row2.float(), atol=1e-6, name="row loss")
+    if d.dtype == torch.float32:
+        at_target = d[torch.arange(N), dev(t)].cpu()
+        want = d2[torch.arange(N), t]
+        # p itself is an fp32 number next to 1: a handful of units in its last place (6e-8 each: the hardware exp2, the sum, the quotient), times 1/N,
+        # is what (p - 1)/N can be known to; the relative bar covers everything above that
+        excess = (at_target - want).abs() - (1e-5 * want.abs() + 5e-7 / N)
+        worst = int(excess.argmax())
+        assert excess[worst] <= 0, (f"gradient at the target column: row {worst} got {at_target[worst].item():.6e} "
+                                    f"want {want[worst].item():.6e}")
+    assert_close(d, d2, atol=5e-7 / N if d.dtype == torch.float32 else 1e-10, name="dlogits")
 
 
 def test_cross_entropy_all_ignored_and_bad_targets(ops):
