@@ -253,6 +253,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   VecE<T, EPV> cur[VPT];
   int64_t tgt = 0;
   bool live = false;
+  float x_t = 0.f;
   if (row < N) {
     tgt = targets[row];
     live = target_counts(tgt, V, ignore_index);
@@ -263,6 +264,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
         const int idx = tid + BLOCK * j;
         if (idx < nvec) cur[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
       }
+      if (tid == 0) x_t = to_acc(x[tgt]);
     }
   }
   int parity = 0;
@@ -272,6 +274,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     VecE<T, EPV> nxt[VPT];
     int64_t ntgt = 0;
     bool nlive = false;
+    float nx_t = 0.f;
     if (nrow < N) {
       ntgt = targets[nrow];
       nlive = target_counts(ntgt, V, ignore_index);
@@ -282,6 +285,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
           const int idx = tid + BLOCK * j;
           if (idx < nvec) nxt[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
         }
+        if (tid == 0) nx_t = to_acc(x[ntgt]);
       }
     }
 
@@ -295,12 +299,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
           store_out<T, TD, VN>(dlogits + row * row_stride + (int64_t)idx * VN, z);
       }
     } else {
-      // the target column sits in vector t_vec = j_t * BLOCK + tid_t, element t_sub: a uniform
-      // test on j and a per-lane element index keep its handling out of the other vectors
-      const int t_vec = (int)(tgt / VN);
-      const int j_t = t_vec / BLOCK;
-      const int my_sub = (t_vec % BLOCK) == tid ? (int)(tgt % VN) : -1;
-      float x_t = 0.f;  // the target's logit, in the lane that holds it
       // ---- widen, mask what is not a class column to -inf, lane-local max
       float e[VPT][VN];
       float m = -INFINITY;
@@ -319,10 +317,6 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
             e[j][k] = c0 + k < iV ? to_acc(cur[j].e[k]) : -INFINITY;
             m = fmaxf(m, e[j][k]);
           }
-        }
-        if (j == j_t) {  // uniform
-#pragma unroll
-          for (int k = 0; k < VN; ++k) x_t = k == my_sub ? e[j][k] : x_t;
         }
       }
       // a lane without any class column: any finite stand-in keeps 2^(-inf - m) = 0
@@ -351,17 +345,14 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
       const float log2_S = __builtin_amdgcn_logf(S);
       // loss = ln(sum exp(x - max)) - (x_t - max), the difference to the maximum formed with one
       // fused multiply-add against the rounded M2 the sum was taken with
-      if (my_sub >= 0 && row_loss) row_loss[row] = (log2_S - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+      if (tid == 0 && row_loss) row_loss[row] = (log2_S - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
 
       if (dlogits) {
         // a lane that holds no class column has e = 0 everywhere; give it f = 0 so that
         // 0 * f cannot meet an overflowed factor
-        // One factor per lane folds the step from the lane's maximum to the row's, 1/sum and
-        // |scale| into a single exponent.  The logarithms in it are good to ~1e-6 relative,
-        // which is fine everywhere except at the target column, where subtracting `scale`
-        // amplifies it when p is close to 1: that one element is formed as a product instead.
         float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml2 - M2 - log2_S + log2_scale);
         f = negate ? -f : f;
+        const int t_vec = (int)(tgt / VN), t_sub = (int)(tgt % VN);
         TD *d = dlogits + row * row_stride;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
@@ -370,10 +361,14 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
             float o[VN];
 #pragma unroll
             for (int k = 0; k < VN; ++k) o[k] = e[j][k] * f;
-            if (j == j_t) {  // uniform
+            if (idx == t_vec) {
+              // the exponent-folded factor f is good to ~1e-6 relative (its logarithms are),
+              // which subtracting `scale` amplifies when p is close to 1: the target element
+              // is formed as a product instead
               const float exact = __builtin_amdgcn_exp2f(ml2 - M2) * (scale * __builtin_amdgcn_rcpf(S));
 #pragma unroll
-              for (int k = 0; k < VN; ++k) o[k] = k == my_sub ? e[j][k] * exact - scale : o[k];
+              for (int k = 0; k < VN; ++k)
+                if (k == t_sub) o[k] = e[j][k] * exact - scale;
             }
             store_out<T, TD, VN>(d + (int64_t)idx * VN, o);
           }
@@ -384,6 +379,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     for (int j = 0; j < VPT; ++j) cur[j] = nxt[j];
     live = nlive;
     tgt = ntgt;
+    x_t = nx_t;
     row = nrow;
   }
 }

@@ -98,10 +98,14 @@ __device__ __forceinline__ float gelu_tanh_bwd_fast(float dy, float x) {
   // d/dx = s * (1 + 2 x (1 - s) kBeta (1 + 3 kKappa x^2))
   constexpr float C0 = (float)(2.0 * kBeta);
   constexpr float C1 = (float)(6.0 * kBeta * kKappa);
-  const float x_sq = x * x;
-  const float s = tanh_gate(x, x_sq);
+  // beyond |x| = 12 the derivative is 1 or 0 to the last bit already; evaluating it at the
+  // clamped point keeps x^3 from overflowing into 0 * inf for |x| > 7e12.  A NaN input stays NaN.
+  const float xc = __builtin_fminf(__builtin_fmaxf(x, -12.0f), 12.0f);
+  const float x_sq = xc * xc;
+  const float s = tanh_gate(xc, x_sq);
   const float inner_d2 = C0 + C1 * x_sq;
-  return dy * (s * (1.0f + x * (1.0f - s) * inner_d2));
+  const float d = s * (1.0f + xc * (1.0f - s) * inner_d2);
+  return dy * (x != x ? x : d);
 }
 
 // Exact (erf) form for 16-bit data.  libm's erff costs more VALU time than the memory

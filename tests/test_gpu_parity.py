@@ -236,6 +236,23 @@ def test_gelu_edge_values(ops, co):
             assert got[8] == float("inf")  # gelu(+inf) = +inf; gelu(-inf) is 0 * inf in ATen's form (NaN)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mode", ["none", "tanh"])
+def test_gelu_every_16_bit_pattern(ops, co, mode, dtype):
+    """All 65536 bit patterns of the storage type, forward and backward: finite inputs against the
+    oracle, NaN in -> NaN out.  (Beyond |x| = 1e18 the reference's tanh derivative overflows into
+    0 * inf = NaN where the value is 0 or 1; those are not compared.)"""
+    x = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    ok = torch.isfinite(x.float()) & (x.float().abs() < 1e18)
+    y, y2 = ops.gelu_forward(dev(x), mode).cpu(), co.gelu_forward(x, mode)
+    assert_close(y[ok], y2[ok], atol=1e-6, name="forward")
+    d, d2 = ops.gelu_backward(dev(torch.ones_like(x)), dev(x), mode).cpu(), co.gelu_backward(torch.ones_like(x), x, mode)
+    assert_close(d[ok], d2[ok], atol=5e-6, name="backward")
+    nan_in = torch.isnan(x.float())
+    assert torch.isnan(y[nan_in].float()).all() and torch.isnan(d[nan_in].float()).all()
+    assert not torch.isnan(d[ok].float()).any()
+
+
 def test_gelu_config3_full_size(ops, co):
     x = randn((8192, 3072), 1340, std=1.5, dtype=torch.bfloat16)
     dy = randn((8192, 3072), 1341, dtype=torch.bfloat16)
