@@ -44,6 +44,10 @@ struct CS_API AdamW {
     // example/gpt2/gpt2_single_device.cpp:706): module::AdamW clips the global gradient norm to
     // this value inside its step.
     CS_ARG(c10::optional<double>, max_grad_norm) = {};
+    // example/gpt2/gpt2_single_device.cpp:619 sets `.fused(true)`, an option the reference's own
+    // header does not declare; it is accepted here so that the example builds.  module::AdamW
+    // updates all parameters in one launch either way.
+    CS_ARG(bool, fused) = true;
   };
 
   static std::shared_ptr<State> init(const Scheduler &scheduler, const ReadOnlyTensor &parameter,
