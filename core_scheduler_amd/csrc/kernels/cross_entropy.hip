@@ -384,6 +384,169 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   }
 }
 
+// Rows too wide for registers (more than 8192 16-byte vectors: vocabularies beyond 65536 at 16
+// bit, 32768 at fp32), and rows whose stride is not a multiple of the vector width (a
+// vocabulary used unpadded).  Persistent workgroups walk rows.  A row is split into a head of
+// single elements up to the first 16-byte boundary, a body of whole vectors and a tail; the
+// base pointers are 16-byte aligned, so gradient rows split at the same columns.  The body is
+// read twice in chunks of kWideU vectors per lane: the first sweep keeps a running (max, sum)
+// per lane (rescaling the sum when the maximum moves: one exp2 per element plus one per
+// chunk), the second sweep re-reads the row, which the first one left in the L2 / last-level
+// cache, and writes the gradient.  Only a handful of scalars is carried between the sweeps,
+// so two workgroups share a CU and cover each other's waits.
+constexpr int kWideU = 2;  // 16-byte vectors per lane and chunk
+static_assert(kWideU == 2, "the chunk sum below adds two vector sums");
+
+template <typename T, typename TD, int BLOCK>
+__global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
+    const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
+    const int *__restrict__ ws_count, int64_t N, int64_t V, int64_t row_stride,
+    int64_t ignore_index, int reduction, float dloss) {
+  constexpr int VN = Vec16<T>::n;
+  constexpr int kWaves = BLOCK / kWave;
+  constexpr int kTailLane = 32;  // lanes [0, VN) own head elements, [32, 32 + VN) tail elements
+  static_assert(VN <= kTailLane, "head and tail lanes overlap");
+  __shared__ float red_m[kWaves], red_s[kWaves];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int stride = (int)row_stride;  // the host checks that it fits
+  const int vcols = (int)V;
+  float scale = dloss;
+  if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
+
+  for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
+    const int64_t tgt = targets[row];
+    const T *x = logits + row * row_stride;
+    TD *d = dlogits ? dlogits + row * row_stride : nullptr;
+    // columns [0, head) before the first aligned vector, nvec vectors, then the rest
+    int head = (int)((VN - (row * row_stride) % VN) % VN);
+    head = head < stride ? head : stride;
+    const int nvec = (stride - head) / VN;
+    const int tail0 = head + nvec * VN;
+    int ecol = -1;  // the single element this lane owns, if any
+    if (tid < head) ecol = tid;
+    if (tid >= kTailLane && tail0 + (tid - kTailLane) < stride) ecol = tail0 + (tid - kTailLane);
+    const T *xb = x + head;
+    TD *db = d ? d + head : nullptr;
+
+    if (!target_counts(tgt, V, ignore_index)) {  // block-uniform
+      if (tid == 0 && row_loss) row_loss[row] = 0.f;
+      if (d) {
+        float z[VN];
+#pragma unroll
+        for (int k = 0; k < VN; ++k) z[k] = 0.f;
+        for (int idx = tid; idx < nvec; idx += BLOCK) store_out<T, TD, VN>(db + (int64_t)idx * VN, z);
+        if (ecol >= 0) d[ecol] = from_acc<TD>(0.f);
+      }
+      continue;
+    }
+    // ---- sweep 1: running maximum (times log2 e) and the sum relative to it
+    float xe = -INFINITY;
+    if (ecol >= 0 && ecol < vcols) xe = to_acc(x[ecol]);
+    float m2 = xe * kLog2e;
+    // the same expression as in the second sweep (the fma sees the product unrounded, so this is not exactly 1)
+    float s = xe == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(xe, kLog2e, -m2));
+    for (int base = tid; base < nvec + tid; base += BLOCK * kWideU) {
+      Vec16<T> v[kWideU];
+#pragma unroll
+      for (int u = 0; u < kWideU; ++u) {
+        const int idx = base + BLOCK * u;
+        if (idx < nvec) v[u] = load16(xb + (int64_t)idx * VN);  // cached: read again below
+      }
+      float xs[kWideU][VN];
+      float cm = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < kWideU; ++u) {
+        const int idx = base + BLOCK * u;
+        const int c0 = head + idx * VN;
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          xs[u][k] = (idx < nvec && c0 + k < vcols) ? vec_get(v[u], k) : -INFINITY;  // padding, lanes past the row
+          cm = fmaxf(cm, xs[u][k]);
+        }
+      }
+      const float cm2 = cm * kLog2e;
+      if (cm2 > m2) {
+        s *= __builtin_amdgcn_exp2f(m2 - cm2);  // 0 the first time (m2 = -inf, s = 0)
+        m2 = cm2;
+      }
+      if (m2 != -INFINITY) {
+        // pairwise within the chunk, one add onto the running sum: once a dominant term sits
+        // in s, every further add rounds at its size, so there should be few of them
+        float part[kWideU];
+#pragma unroll
+        for (int u = 0; u < kWideU; ++u) {
+          float e[VN];
+#pragma unroll
+          for (int k = 0; k < VN; ++k) e[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(xs[u][k], kLog2e, -m2));
+#pragma unroll
+          for (int w = VN / 2; w > 0; w /= 2)
+#pragma unroll
+            for (int k = 0; k < w; ++k) e[k] += e[k + w];
+          part[u] = e[0];
+        }
+        s += part[0] + part[1];
+      }
+    }
+    // ---- (max, sum) across the wave, then across the waves
+    const float mw2 = wave_reduce(m2, MaxOp{});
+    const float sw = wave_reduce(m2 == -INFINITY ? 0.f : s * __builtin_amdgcn_exp2f(m2 - mw2), SumOp{});
+    __syncthreads();  // the previous row's readers are done with red_m / red_s
+    if (lane == 0) {
+      red_m[wave] = mw2;
+      red_s[wave] = sw;
+    }
+    __syncthreads();
+    const float pm = lane < kWaves ? red_m[lane] : -INFINITY;
+    const float ps = lane < kWaves ? red_s[lane] : 0.f;
+    const float M2 = wave_reduce(pm, MaxOp{});
+    const float S = wave_reduce(pm == -INFINITY ? 0.f : ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
+    if (tid == 0 && row_loss) {
+      const float x_t = to_acc(x[tgt]);
+      row_loss[row] = (__builtin_amdgcn_logf(S) - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+    }
+    if (!d) continue;
+    // ---- sweep 2: p = 2^(x log2e - M2) / S, gradient (p - onehot) * scale
+    const float factor = scale / S;
+    const int t_vec = tgt >= head ? (int)((tgt - head) / VN) : -1;  // past the body if in the tail
+    const int t_sub = (int)((tgt - head) % VN);
+    if (ecol >= 0) {
+      float o = 0.f;
+      if (ecol < vcols) {
+        o = __builtin_amdgcn_exp2f(__builtin_fmaf(xe, kLog2e, -M2)) * factor;
+        if (ecol == tgt) o -= scale;
+      }
+      d[ecol] = from_acc<TD>(o);
+    }
+    for (int base = tid; base < nvec + tid; base += BLOCK * kWideU) {
+      Vec16<T> v[kWideU];
+#pragma unroll
+      for (int u = 0; u < kWideU; ++u) {
+        const int idx = base + BLOCK * u;
+        if (idx < nvec) v[u] = load16_stream(xb + (int64_t)idx * VN);
+      }
+#pragma unroll
+      for (int u = 0; u < kWideU; ++u) {
+        const int idx = base + BLOCK * u;
+        if (idx < nvec) {
+          const int c0 = head + idx * VN;
+          float o[VN];
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            o[k] = c0 + k < vcols ? __builtin_amdgcn_exp2f(__builtin_fmaf(vec_get(v[u], k), kLog2e, -M2)) * factor : 0.f;
+          if (idx == t_vec) {
+#pragma unroll
+            for (int k = 0; k < VN; ++k)
+              if (k == t_sub) o[k] -= scale;
+          }
+          store_out<T, TD, VN>(db + (int64_t)idx * VN, o);
+        }
+      }
+    }
+  }
+}
+
 // Any V, stride and alignment; fp64 too.  Three sweeps over the row, the
 // later ones served by the cache.
 template <typename T, typename TD>
@@ -443,13 +606,35 @@ int64_t compute_units() {
   return cached[dev];
 }
 
+// Two-sweep kernel: workgroups of 1024 lanes, two per CU, for wide rows; of 256 lanes, eight
+// per CU, where a row has too few vectors to occupy 1024.
+template <typename T, typename TD>
+void launch_wide(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
+                 const int *ws_count, int64_t N, int64_t V, int64_t row_stride, int64_t ignore_index,
+                 int reduction, float dloss, hipStream_t s) {
+  const int64_t cus = compute_units();
+  const int64_t nvec = row_stride / Vec16<T>::n;
+  if (nvec > 256 * kWideU * 2) {
+    const dim3 grid((unsigned)(N < 2 * cus ? N : 2 * cus));
+    ce_rows_wide_kernel<T, TD, 1024><<<grid, dim3(1024), 0, s>>>(
+        (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
+        reduction, dloss);
+  } else {
+    const dim3 grid((unsigned)(N < 8 * cus ? N : 8 * cus));
+    ce_rows_wide_kernel<T, TD, 256><<<grid, dim3(256), 0, s>>>(
+        (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
+        reduction, dloss);
+  }
+}
+
 template <typename T, typename TD>
 int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
                 const int *ws_count, int64_t N, int64_t V, int64_t row_stride,
                 int64_t ignore_index, int reduction, float dloss, hipStream_t s) {
   constexpr int VN = Vec16<T>::n;
-  const bool vec_ok = !std::is_same_v<T, double> && row_stride % VN == 0 && is_aligned16(logits) &&
-                      (!dlogits || is_aligned16(dlogits)) && row_stride / VN <= 1024 * 16;
+  const bool base_ok = !std::is_same_v<T, double> && is_aligned16(logits) &&
+                       (!dlogits || is_aligned16(dlogits)) && row_stride <= (int64_t(1) << 30);
+  const bool vec_ok = base_ok && row_stride % VN == 0;
   const dim3 grid((unsigned)N);
   if constexpr (!std::is_same_v<T, double>) {
     if (vec_ok) {
@@ -462,8 +647,10 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         CS_CE(64, 8);
       } else if (nvec <= 256 * 8) {
         CS_CE(256, 8);
-      } else if (nvec <= 1024 * 8) {
-        // one persistent workgroup per CU
+      } else if (nvec <= (sizeof(T) == 4 ? 1024 * 8 : sizeof(TD) == 4 ? 512 * 13 : 1024 * 7)) {
+        // one persistent workgroup per CU, the row in registers.  The widest plans (8 vectors
+        // per lane at 16 bit, 16 half vectors with fp32 gradients) measured slower than the
+        // two-sweep kernel and are not built.
         const int64_t cus = compute_units();
         const dim3 pgrid((unsigned)(N < cus ? N : cus));
 #define CS_CE_STREAM(VPT, EPV)                                                              \
@@ -471,22 +658,26 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
       (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,      \
       ignore_index, reduction, dloss)
         if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
-          // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
-          if (nvec * 2 <= 1024 * 13) {
-            CS_CE_STREAM(13, 4);
-          } else {
-            CS_CE_STREAM(16, 4);
-          }
+          CS_CE_STREAM(13, 4);  // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
         } else if (nvec <= 1024 * 7) {
           CS_CE_STREAM(7, VN);
         } else {
-          CS_CE_STREAM(8, VN);
+          if constexpr (sizeof(T) == 4) CS_CE_STREAM(8, VN);
         }
 #undef CS_CE_STREAM
+      } else if (sizeof(T) == 4 && nvec <= 1024 * 16) {
+        CS_CE(1024, 16);  // fp32 rows up to 65536 columns still fit in registers
       } else {
-        CS_CE(1024, 16);
+        launch_wide<T, TD>(logits, dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
+                           reduction, dloss, s);
       }
 #undef CS_CE
+      return launch_status();
+    }
+    if (base_ok && sizeof(TD) >= sizeof(T)) {
+      // rows that start off a 16-byte boundary: split per row into head, vectors and tail
+      launch_wide<T, TD>(logits, dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
+                         reduction, dloss, s);
       return launch_status();
     }
   }
