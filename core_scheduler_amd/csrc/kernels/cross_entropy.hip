@@ -21,6 +21,7 @@
 
 #include <math.h>
 
+#include <atomic>
 #include <type_traits>
 
 namespace cs_hip {
@@ -592,18 +593,19 @@ __global__ __launch_bounds__(256) void ce_rows_general_kernel(
   }
 }
 
-// CUs of the current device, asked once per device.
+// CUs of the current device, asked once per device (threads may race to fill a slot: they
+// store the same value).
 int64_t compute_units() {
-  static int cached[64] = {0};
+  static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
       n = 256;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 
 // Two-sweep kernel: workgroups of 1024 lanes, two per CU, for wide rows; of 256 lanes, eight

@@ -32,6 +32,7 @@
 // read of dout and a second write of the indexed rows.
 #include "common.cuh"
 
+#include <atomic>
 #include <type_traits>
 
 namespace cs_hip {
@@ -768,14 +769,14 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
 // The reduce kernel's dynamic LDS can exceed the 64 KB a launch gets by default (wide windows).
 template <typename T>
 int allow_reduce_lds(size_t bytes) {
-  static bool done[64] = {false};
+  static std::atomic<bool> done[64];  // bytes is one constant per T; racing threads set the same value
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
-  if (!done[dev]) {
+  if (!done[dev].load(std::memory_order_acquire)) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&emb_bwd_reduce_kernel<T>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) return (int)e;
-    done[dev] = true;
+    done[dev].store(true, std::memory_order_release);
   }
   return CS_OK;
 }
