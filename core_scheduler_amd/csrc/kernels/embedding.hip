@@ -328,6 +328,110 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
   sorted_pos[rank] = KeyCodec<KeyT>::pos(key, shift);
 }
 
+// -------------------------------------------- backward: ranking a short list
+// With few enough keys (they all fit in the LDS of one workgroup) sorting takes one launch
+// instead of two: a key's place in the sorted order is the number of keys below it (keys are
+// distinct: they contain the position), found by comparing it with every other key.  That is
+// n^2 comparisons, 2 VALU operations each and nothing else, spread evenly over the chip, next
+// to the zero fill that the same launch does.
+//
+// A workgroup of 1024 lanes ranks kRankOwn = 32 keys.  It first builds every key of the list
+// in its LDS.  Lane l then owns key (l mod 32) of the workgroup's 32 and belongs to one of
+// 32 groups; group g compares against the 16-byte key quads g, g + 32, g + 64, ...: the two
+// groups of a wave read adjacent quads (no bank conflict, every lane of a group the same
+// address).  The 32 partial counts of a key are added through the LDS.
+// Launch layout, in block order (the ranking workgroups run longest, so they start first):
+//   [0, rank_blocks)            rank 32 keys each; also preset the unused tail of sorted_id
+//   + pos_blocks                position-table gradient, 1024 vectors per block
+//   + the rest                  zero fill of fill_dst[0, fill_vecs)
+constexpr int kRankThreads = 1024;
+constexpr int kRankOwn = 32;
+constexpr int kRankGroups = kRankThreads / kRankOwn;
+#ifndef CS_EMB_RANK_MAX_KEY_BYTES
+#define CS_EMB_RANK_MAX_KEY_BYTES 32768
+#endif
+constexpr size_t kRankMaxKeyBytes = CS_EMB_RANK_MAX_KEY_BYTES;  // longest key list that is ranked this way
+constexpr size_t kRankPartBytes = (size_t)kRankGroups * kRankOwn * sizeof(int);
+
+template <typename KeyT, typename IdxT, typename T>
+__global__ __launch_bounds__(kRankThreads) void emb_bwd_rank_kernel(
+    const IdxT *__restrict__ ids, uint32_t *__restrict__ sorted_id,
+    uint32_t *__restrict__ sorted_pos, int64_t n, int n_quads, int shift, int64_t num_weights,
+    int64_t padding_idx, const T *__restrict__ dout, T *__restrict__ dwpe, int64_t B, int64_t TC,
+    int accumulate, int rank_blocks, int64_t pos_blocks, u32x4 *__restrict__ fill_dst,
+    int64_t fill_vecs) {
+  typedef KeyT Quad __attribute__((ext_vector_type(4)));
+  extern __shared__ u32x4 rank_lds[];
+  __shared__ int valid_of_wave[kRankThreads / kWave];
+  const int tid = threadIdx.x;
+  const int64_t blk = blockIdx.x;
+  if (blk >= rank_blocks + pos_blocks) {
+    zero_fill_block<kRankThreads>(fill_dst, fill_vecs, blk - rank_blocks - pos_blocks, tid);
+    return;
+  }
+  if (blk >= rank_blocks) {
+    const int64_t f = (blk - rank_blocks) * kRankThreads + tid;
+    if (f < TC / Vec16<T>::n) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
+    return;
+  }
+  KeyT *keys = reinterpret_cast<KeyT *>(rank_lds);  // [4 n_quads], padded with sentinels
+  int *part = reinterpret_cast<int *>(keys + (size_t)n_quads * 4);  // [kRankGroups][kRankOwn]
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int n_keys = n_quads * 4;
+
+  // ---- every key of the list, and how many are real
+  int mine = 0;
+  for (int i = tid; i < n_keys; i += kRankThreads) {
+    KeyT key = KeyCodec<KeyT>::kSentinel;
+    if (i < n) {
+      const int64_t id = (int64_t)ids[i];
+      if (id >= 0 && id < num_weights && id != padding_idx)
+        key = KeyCodec<KeyT>::make((uint32_t)id, (uint32_t)i, shift);
+    }
+    keys[i] = key;
+    mine += key != KeyCodec<KeyT>::kSentinel ? 1 : 0;
+  }
+  const int in_wave = wave_reduce(mine, SumOp{});
+  if (lane == 0) valid_of_wave[wave] = in_wave;
+  __syncthreads();
+  int n_valid = 0;
+#pragma unroll
+  for (int w = 0; w < kRankThreads / kWave; ++w) n_valid += valid_of_wave[w];
+
+  // ---- entries past the real keys read "no id": each ranking workgroup presets a share
+  {
+    const int tail = (int)n - n_valid;
+    const int share = (tail + rank_blocks - 1) / rank_blocks;
+    for (int i = tid; i < share; i += kRankThreads) {
+      const int64_t at = (int64_t)n_valid + blk * share + i;
+      if (at < n) sorted_id[at] = kNoId;
+    }
+  }
+
+  // ---- partial counts
+  const int slot = lane & (kRankOwn - 1);
+  const int group = wave * (kWave / kRankOwn) + lane / kRankOwn;
+  const int own_at = (int)blk * kRankOwn + slot;
+  const KeyT own = own_at < n_keys ? keys[own_at] : KeyCodec<KeyT>::kSentinel;
+  const Quad *quads = reinterpret_cast<const Quad *>(keys);
+  int below = 0;
+#pragma unroll 4
+  for (int q = group; q < n_quads; q += kRankGroups) {
+    const Quad k = quads[q];
+    below += (k.x < own ? 1 : 0) + (k.y < own ? 1 : 0) + (k.z < own ? 1 : 0) + (k.w < own ? 1 : 0);
+  }
+  part[group * kRankOwn + slot] = below;
+  __syncthreads();
+  if (tid < kRankOwn && own != KeyCodec<KeyT>::kSentinel) {
+    int rank = 0;
+#pragma unroll
+    for (int g = 0; g < kRankGroups; ++g) rank += part[g * kRankOwn + tid];
+    sorted_id[rank] = KeyCodec<KeyT>::id(own, shift);
+    sorted_pos[rank] = KeyCodec<KeyT>::pos(own, shift);
+  }
+}
+
 // ------------------------------------------------------ backward: reduction
 constexpr int kOwn = 4;                         // sorted entries per wave
 constexpr int kRedWaves = kWindow / kOwn;       // 8
@@ -736,6 +840,27 @@ int fwd_dispatch(const void *weight, const void *wpe, const void *ids, void *out
   return CS_ERR_UNSUPPORTED;
 }
 
+// Kernels whose dynamic LDS can exceed the 64 KB a launch gets by default ask for their maximum
+// once per device.  `bytes` is one constant per kernel, so racing threads set the same value;
+// `done` is that kernel's array of per-device flags.
+int allow_dynamic_lds_once(const void *kernel, size_t bytes, std::atomic<bool> *done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  if (!done[dev].load(std::memory_order_acquire)) {
+    const hipError_t e =
+        hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+    done[dev].store(true, std::memory_order_release);
+  }
+  return CS_OK;
+}
+template <typename KeyT, typename IdxT, typename T>
+int allow_rank_lds(size_t bytes) {
+  static std::atomic<bool> done[64];
+  return allow_dynamic_lds_once(
+      reinterpret_cast<const void *>(&emb_bwd_rank_kernel<KeyT, IdxT, T>), bytes, done);
+}
+
 // Sort + merge.  The sort launch also sums dwpe (`fused_positions`), and both launches clear
 // their share of fill_dst[0, fill_vecs), on the CUs the sorting leaves idle.
 template <typename KeyT, typename IdxT, typename T>
@@ -746,8 +871,23 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   uint32_t *sorted_id = reinterpret_cast<uint32_t *>(ws + L.off_sorted_id);
   uint32_t *sorted_pos = reinterpret_cast<uint32_t *>(ws + L.off_sorted_pos);
   const int64_t pos_blocks = fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)kTile) : 0;
-  // whole fill workgroups to the sort launch, the remainder to the merge launch
   const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecs);
+  const int64_t n_quads = ceil_div(n, (int64_t)4);
+  if ((size_t)n_quads * 4 * sizeof(KeyT) <= kRankMaxKeyBytes) {
+    // a short list: one launch ranks every key against all others
+    static_assert(kRankThreads == kTile, "the position blocks cover kTile vectors each");
+    const int64_t rank_blocks = ceil_div(n_quads * 4, (int64_t)kRankOwn);
+    const int64_t blocks = rank_blocks + pos_blocks + fill_blocks;
+    if (blocks == 0) return CS_OK;
+    const size_t lds = (size_t)n_quads * 4 * sizeof(KeyT) + kRankPartBytes;
+    const int st = allow_rank_lds<KeyT, IdxT, T>(kRankMaxKeyBytes + kRankPartBytes);
+    if (st != CS_OK) return st;
+    emb_bwd_rank_kernel<KeyT, IdxT, T><<<dim3((unsigned)blocks), dim3(kRankThreads), lds, s>>>(
+        (const IdxT *)ids, sorted_id, sorted_pos, n, (int)n_quads, L.shift, num_weights, padding_idx,
+        dout, dwpe, B, TC, accumulate, (int)rank_blocks, pos_blocks, fill_dst, fill_vecs);
+    return launch_status();
+  }
+  // whole fill workgroups to the sort launch, the remainder to the merge launch
   const int64_t sort_fill_blocks = fill_blocks * CS_EMB_FILL_SORT_PCT / 100;
   const int64_t sort_fill_vecs =
       sort_fill_blocks * kFillVecs < fill_vecs ? sort_fill_blocks * kFillVecs : fill_vecs;
@@ -766,19 +906,10 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   return launch_status();
 }
 
-// The reduce kernel's dynamic LDS can exceed the 64 KB a launch gets by default (wide windows).
 template <typename T>
 int allow_reduce_lds(size_t bytes) {
-  static std::atomic<bool> done[64];  // bytes is one constant per T; racing threads set the same value
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
-  if (!done[dev].load(std::memory_order_acquire)) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&emb_bwd_reduce_kernel<T>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return (int)e;
-    done[dev].store(true, std::memory_order_release);
-  }
-  return CS_OK;
+  static std::atomic<bool> done[64];
+  return allow_dynamic_lds_once(reinterpret_cast<const void *>(&emb_bwd_reduce_kernel<T>), bytes, done);
 }
 
 template <typename T>
