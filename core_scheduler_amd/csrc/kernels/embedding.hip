@@ -28,6 +28,9 @@
 //                   a hot row is read by as many CUs as it has windows.
 //   4. finish     - the workgroup of a crossing segment's first window adds
 //                   that segment's partial rows in window order.
+// A list of at most 8192 entries skips 1 and 2: one launch ranks every key by
+// comparing it with all others (see emb_bwd_rank_kernel), and does the zero
+// fill and the position-table sum next to that.
 // The traffic that matters is the dense write of dweight (V*C elements), one
 // read of dout and a second write of the indexed rows.
 #include "common.cuh"
@@ -461,6 +464,10 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
   // ---- ids of the window (lane l <-> entry p0 + l), the entry before and the entry after
   const int64_t p = p0 + lane;
   const bool in_window = lane < kWindow;
+  // lanes 0..3: the positions of this wave's four entries, asked for together with the ids
+  // (an entry past the real ones holds no position; it is never used)
+  const int64_t own_p = p0 + wave * kOwn + lane;
+  const uint32_t lane_pos = (lane < kOwn && own_p < n) ? sorted_pos[own_p] : 0u;
   const uint32_t my_id = (in_window && p < n) ? sorted_id[p] : kNoId;
   const uint32_t prev_id = (in_window && p > 0 && p <= n) ? sorted_id[p - 1] : kNoId;
   const uint64_t valid = __ballot(my_id != kNoId);
@@ -485,8 +492,6 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
     // ---- level 1: this wave's four entries
     const int e0 = wave * kOwn;
     Vec16<T> r[kOwn][kVpl];
-    // lanes 0..3 fetch the four positions together; the rows are then loaded at once
-    const uint32_t lane_pos = (lane < kOwn && e0 + lane < n_valid) ? sorted_pos[p0 + e0 + lane] : 0u;
 #pragma unroll
     for (int e = 0; e < kOwn; ++e) {
       if (e0 + e < n_valid) {
