@@ -482,7 +482,11 @@ def test_embedding_backward_reference_test_case(ops, co, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
 @pytest.mark.parametrize("n,V,C", [(1, 5, 8), (8, 5, 8), (9, 40, 16), (2048, 300, 64), (2049, 1000, 72),
-                                   (5000, 7, 128), (4097, 100000, 8), (300, 50, 12), (64, 20, 7)])
+                                   (5000, 7, 128), (4097, 100000, 8), (300, 50, 12), (64, 20, 7),
+                                   # 64-bit sort keys (V * padded n >= 2^32): ranked in one launch / tile-sorted
+                                   (3000, 2000000, 8), (5000, 2000000, 8),
+                                   # 32-bit keys either side of the longest list that is ranked in one launch
+                                   (8192, 3000, 16), (8193, 3000, 16), (20000, 50, 8)])
 def test_embedding_backward_shapes(ops, co, dtype, n, V, C):
     ids = randint(0, V, (n,), 92)
     dout = randn((n, C), 93, dtype=dtype)
