@@ -297,6 +297,9 @@ int cs_embedding_backward_positions(const void *dout, void *dwpe, int64_t B,
  * for MEAN and dloss otherwise; padding columns are written as zero.  The
  * reference has no upstream gradient (it passes ones_like(loss)):
  * dloss = 1 reproduces it.
+ * Any row_stride >= V is accepted.  Rows that start on 16-byte boundaries
+ * and have at most 57344 columns (16 bit) or 65536 (fp32) are read once;
+ * other rows are read twice, the second time from cache.
  * ---------------------------------------------------------------------- */
 size_t cs_fused_classifier_workspace_bytes(int64_t N);
 int cs_fused_classifier(const void *logits, void *dlogits,
