@@ -98,6 +98,31 @@ def test_embedding_routine(host, sched, co, dtype):
 
 
 @pytest.mark.gpu
+def test_embedding_inside_autocast_guard(host, sched, co):
+    # test/test_autocast.cpp:158-204: fp32 table and fp32 upstream gradient, guard set to bf16;
+    # a gather is not an autocast op, so output and gradient stay fp32
+    B, T, V, d = 2, 1024, 4095, 512
+    ids = randint(0, 3, (B, T), 30, dtype=torch.int32)
+    state = host.Embedding.init(sched, V, d, dtype="float32")
+    w = down(host, sched, state.weight)
+    scope = host.autocast()
+    scope.enter(sched, "bfloat16")
+    try:
+        out = host.Embedding.forward(sched, state, up(host, sched, ids))
+        out.wait()
+    finally:
+        scope.exit()
+    got = down(host, sched, out)
+    assert got.dtype == torch.float32
+    assert_bit_exact(got, co.embedding_forward(w, ids), "forward")
+    dout = randn((B, T, d), 31)
+    host.Embedding.backward(sched, state, up(host, sched, dout))
+    grad = down(host, sched, state.grad_weight)
+    assert grad.dtype == torch.float32
+    assert_close(grad, co.embedding_backward(dout, ids, V), atol=2e-5, name="grad")
+
+
+@pytest.mark.gpu
 def test_embedding_with_positions(host, sched, co):
     B, T, V, C = 4, 64, 500, 128
     tok = host.Embedding.init(sched, V, C, dtype="bfloat16")
