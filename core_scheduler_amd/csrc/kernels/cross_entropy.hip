@@ -330,9 +330,12 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
           e[j][k] = __builtin_amdgcn_exp2f(e[j][k] * kLog2e - ml2);
           s += e[j][k];
         }
-      // ---- (max, sum) across the wave, then across the 16 waves
-      const float mw2 = wave_reduce(ml2, MaxOp{});
-      const float sw = wave_reduce(s * __builtin_amdgcn_exp2f(ml2 - mw2), SumOp{});
+      // ---- (max, sum) across the wave, then across the 16 waves.  A lane without a finite
+      // value takes no part: its stand-in maximum must not pass for a real one (the real ones
+      // may all lie far below it), and its empty sum must not meet an overflowed 2^(0 - max)
+      const bool empty = m == -INFINITY;
+      const float mw2 = wave_reduce(empty ? -INFINITY : ml2, MaxOp{});
+      const float sw = wave_reduce(empty ? 0.f : s * __builtin_amdgcn_exp2f(ml2 - mw2), SumOp{});
       if (lane == 0) {
         red_m[parity][wave] = mw2;
         red_s[parity][wave] = sw;
@@ -341,7 +344,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
       const float pm = lane < kWaves ? red_m[parity][lane] : -INFINITY;
       const float ps = lane < kWaves ? red_s[parity][lane] : 0.f;
       const float M2 = wave_reduce(pm, MaxOp{});
-      const float S = wave_reduce(ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
+      const float S = wave_reduce(pm == -INFINITY ? 0.f : ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
       parity ^= 1;  // the other pair of arrays next time: one barrier per row is enough
       const float log2_S = __builtin_amdgcn_logf(S);
       // loss = ln(sum exp(x - max)) - (x_t - max), the difference to the maximum formed with one
@@ -351,7 +354,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
       if (dlogits) {
         // a lane that holds no class column has e = 0 everywhere; give it f = 0 so that
         // 0 * f cannot meet an overflowed factor
-        float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml2 - M2 - log2_S + log2_scale);
+        float f = empty ? 0.f : __builtin_amdgcn_exp2f(ml2 - M2 - log2_S + log2_scale);
         f = negate ? -f : f;
         const int t_vec = (int)(tgt / VN), t_sub = (int)(tgt % VN);
         TD *d = dlogits + row * row_stride;

@@ -708,6 +708,37 @@ def test_cross_entropy_rows_beyond_registers(ops, co, N, V, stride, dtype, gdt):
     assert none is None and loss3.item() == loss.item()
 
 
+@pytest.mark.parametrize("N,V,stride,dtype,gdt", [(6, 50257, 50304, torch.bfloat16, None),
+                                                   (6, 50257, 50304, torch.bfloat16, torch.float32),
+                                                   (6, 50257, 50304, torch.float32, None),
+                                                   (6, 1000, 1024, torch.float32, None),
+                                                   (6, 70000, 70000, torch.bfloat16, None),
+                                                   (6, 50257, 50257, torch.float16, None),
+                                                   (6, 301, 301, torch.float64, None)])
+def test_cross_entropy_masked_vocabulary(ops, co, N, V, stride, dtype, gdt):
+    """Logits masked with -inf, as when the vocabulary is restricted: whole lanes, waves and
+    vectors without a finite value, next to finite logits far below zero (their exponentials
+    relative to 0 would underflow) or of ordinary size."""
+    x = torch.full((N, stride), float("-inf"), dtype=dtype)
+    g = torch.Generator().manual_seed(122)
+    keep = [slice(0, 100), slice(V - 37, V), slice(V // 2, V // 2 + 3), slice(5, 6), slice(0, V, 97), slice(0, V)]
+    level = [-60.0, -60.0, 50.0, 0.0, -60.0, 0.0]
+    t = torch.zeros(N, dtype=torch.int64)
+    for r in range(N):
+        cols = torch.arange(V)[keep[r]]
+        x[r, cols] = (torch.randn(len(cols), generator=g) * 2 + level[r]).to(dtype)
+        t[r] = cols[len(cols) // 2]
+    x[N - 1, 17:min(4000, V // 3)] = float("-inf")  # a hole in an otherwise ordinary row, clear of its target
+    kw = dict(dlogits_dtype=gdt) if gdt else {}
+    loss, row, d, _ = ops.fused_classifier(dev(x), dev(t), V, **kw)
+    loss2, row2, d2, _ = co.cross_entropy(x, t, V, **kw)
+    assert torch.isfinite(row).all() and torch.isfinite(d.float()).all()
+    assert_close(row, row2.to(row.dtype), atol=1e-5, name="row loss")
+    assert_close(loss, loss2.to(loss.dtype), atol=1e-5, name="loss")
+    assert_close(d, d2, atol=1.2e-7 / N, name="dlogits")
+    assert (d[x.isinf().to(d.device)] == 0).all()
+
+
 def test_cross_entropy_all_ignored_and_bad_targets(ops):
     x = randn((6, 128), 115, dtype=torch.bfloat16)
     t = torch.full((6,), -100, dtype=torch.int64)
