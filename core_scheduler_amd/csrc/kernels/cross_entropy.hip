@@ -662,7 +662,9 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
   ce_rows_stream_kernel<T, TD, VPT, EPV><<<pgrid, dim3(1024), 0, s>>>(                      \
       (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,      \
       ignore_index, reduction, dloss)
-        if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
+        if constexpr (std::is_same_v<T, f16_t> && sizeof(TD) == 4) {
+          CS_CE_STREAM(7, VN);
+        } else if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
           CS_CE_STREAM(13, 4);  // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
         } else if (nvec <= 1024 * 7) {
           CS_CE_STREAM(7, VN);
