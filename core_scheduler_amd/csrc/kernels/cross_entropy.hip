@@ -673,7 +673,8 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         }
 #undef CS_CE_STREAM
       } else if (sizeof(T) == 4 && nvec <= 1024 * 16) {
-        CS_CE(1024, 16);  // fp32 rows up to 65536 columns still fit in registers
+        // fp32 rows up to 65536 columns still fit in registers (at 16 bit this plan spills)
+        if constexpr (sizeof(T) == 4) CS_CE(1024, 16);
       } else {
         launch_wide<T, TD>(logits, dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
                            reduction, dloss, s);
