@@ -9,14 +9,19 @@
 //   loss      = sum_i loss_i / #{not ignored}        (MEAN)  |  sum_i loss_i (SUM)
 //   dlogits_i = (softmax(x_i) - onehot(t_i)) * s,    s = dloss / #{not ignored} (MEAN) | dloss
 //
-// One workgroup owns one row and keeps it in registers as 16-byte vectors
-// (50257 bf16 = 6283 vectors = 7 per lane at 1024 lanes, 28 VGPRs), so the
-// row is read from HBM once and dlogits written once: 2 accesses per
-// element.  The max and the sum of exponentials are exact two-step
-// reductions over registers (wave64 butterfly, then LDS across the 16
-// waves), not a running rescale; the probabilities are formed as
-// 2^(x*log2e - K) with K = max*log2e + log2(sum) - log2(s) folded into one
-// constant, which costs one fma and one hardware exp2 per element.
+// A row is read from HBM once and its gradient written once: 2 accesses per
+// element.  Which kernel does that depends on the row's width:
+//   up to 2048 vectors of 16 bytes   ce_rows_kernel: one workgroup per row, the row in
+//                                    registers, exact two-step max and sum (wave64
+//                                    butterfly, then LDS across the waves)
+//   up to 7168 (8192 at fp32)        ce_rows_stream_kernel: one persistent workgroup per
+//                                    CU that loads the next row while it works on the
+//                                    current one (50257 bf16 = 6283 vectors = 7 per lane)
+//   wider, or rows that do not       ce_rows_wide_kernel: two sweeps over the row, the
+//   start on 16-byte boundaries      second one served by the cache
+//   fp64, unaligned base pointers    ce_rows_general_kernel
+// Probabilities are 2^(x*log2e - max*log2e) / sum with one fma and one hardware exp2 per
+// element; the row loss is ln(sum) - (x_t - max).
 #include "common.cuh"
 
 #include <math.h>
