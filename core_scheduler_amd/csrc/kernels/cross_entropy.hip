@@ -223,6 +223,28 @@ __device__ __forceinline__ VecE<T, EPV> load_e_stream(const T *p) {
   }
 }
 
+// Element k of v as fp32.  fp16 is converted straight out of its half of the 32-bit register
+// (the sub-dword select of the conversion instruction): shifting the upper half down first
+// costs a temporary register per element, which the 13 x 4 plan does not have (the plans with
+// 16-byte loads have, and keep the compiler's own sequence).
+template <typename T, int EPV>
+__device__ __forceinline__ float widen(const VecE<T, EPV> &v, int k) {
+  if constexpr (std::is_same_v<T, f16_t> && EPV == 4) {
+    typedef uint32_t words_t __attribute__((ext_vector_type(EPV / 2)));
+    const words_t w = __builtin_bit_cast(words_t, v);
+    const uint32_t word = w[k >> 1];
+    float f;
+    if (k & 1) {
+      asm("v_cvt_f32_f16_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1" : "=v"(f) : "v"(word));
+    } else {
+      asm("v_cvt_f32_f16_e32 %0, %1" : "=v"(f) : "v"(word));
+    }
+    return f;
+  } else {
+    return to_acc(v.e[k]);
+  }
+}
+
 // Streaming variant for wide rows (the GPT-2 vocabulary): one 1024-lane
 // workgroup per CU walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and
 // loads the next row into a second register set before it starts on the
@@ -314,13 +336,13 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
         if (c0 + VN <= iV) {
 #pragma unroll
           for (int k = 0; k < VN; ++k) {
-            e[j][k] = to_acc(cur[j].e[k]);
+            e[j][k] = widen(cur[j], k);
             m = fmaxf(m, e[j][k]);
           }
         } else {
 #pragma unroll
           for (int k = 0; k < VN; ++k) {
-            e[j][k] = c0 + k < iV ? to_acc(cur[j].e[k]) : -INFINITY;
+            e[j][k] = c0 + k < iV ? widen(cur[j], k) : -INFINITY;
             m = fmaxf(m, e[j][k]);
           }
         }
@@ -667,9 +689,7 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
   ce_rows_stream_kernel<T, TD, VPT, EPV><<<pgrid, dim3(1024), 0, s>>>(                      \
       (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,      \
       ignore_index, reduction, dloss)
-        if constexpr (std::is_same_v<T, f16_t> && sizeof(TD) == 4) {
-          CS_CE_STREAM(7, VN);
-        } else if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
+        if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
           CS_CE_STREAM(13, 4);  // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
         } else if (nvec <= 1024 * 7) {
           CS_CE_STREAM(7, VN);

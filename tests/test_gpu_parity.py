@@ -632,10 +632,12 @@ def test_cross_entropy_inplace_amp_and_dloss(ops, co):
 
 @pytest.mark.parametrize("N,V,stride", [(300, 50257, 50304), (270, 59990, 60000), (5, 65536, 65536),
                                         (530, 50257, 50257), (70, 999, 1001)])
-def test_cross_entropy_autocast_wide_rows(ops, co, N, V, stride):
-    """16-bit logits with fp32 gradients on the streaming kernel's two register plans, with more
-    rows than workgroups (so rows are prefetched) and ignored rows among them."""
-    x = randn((N, stride), 116, std=2.0, dtype=torch.bfloat16)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cross_entropy_autocast_wide_rows(ops, co, N, V, stride, dtype):
+    """16-bit logits with fp32 gradients on the streaming kernel's register plan and the
+    two-sweep kernel, with more rows than workgroups (so rows are prefetched) and ignored rows
+    among them."""
+    x = randn((N, stride), 116, std=2.0, dtype=dtype)
     t = randint(0, V, (N,), 117)
     t[1] = -100
     t[N - 1] = -100
