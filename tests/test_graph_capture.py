@@ -99,3 +99,43 @@ def test_captured_step_replays_match_eager():
         for a, b, name in zip(got, eager[i], "x y act dlogits row_loss loss dact dx dgamma dbeta dwte dwpe w m v".split()):
             assert_bit_exact(a, b, f"replay {i}: {name}")
         del scratch
+
+
+def test_two_streams_give_the_serial_results():
+    """The library keeps no per-call state of its own: the same ops issued on two streams at once,
+    each with its own buffers and workspaces, give bit for bit what each gives alone."""
+    from core_scheduler_amd import ops
+
+    def work(seed):
+        B, T, C, V = 8, 512, 768, 50257
+        ids = randint(0, V, (B, T), seed).to(DEV)
+        dout = randn((B, T, C), seed + 1, dtype=torch.bfloat16).to(DEV)
+        x = randn((B * T, C), seed + 2, dtype=torch.bfloat16).to(DEV)
+        gamma, beta = randn((C,), seed + 3).to(DEV), randn((C,), seed + 4).to(DEV)
+        logits = randn((512, 50304), seed + 5, std=2.0, dtype=torch.bfloat16).to(DEV)
+        tgt = randint(0, V, (512,), seed + 6).to(DEV)
+        return dict(ids=ids, dout=dout, x=x, gamma=gamma, beta=beta, logits=logits, tgt=tgt, V=V)
+
+    def run(wk):
+        y, mean, rstd = ops.layernorm_forward(wk["x"], wk["gamma"], wk["beta"])
+        dx, dgamma, dbeta = ops.layernorm_backward(wk["dout"].reshape(wk["x"].shape), wk["x"], mean, rstd, wk["gamma"])
+        dwte, dwpe = ops.embedding_backward_fused(wk["dout"], wk["ids"], wk["V"])
+        loss, row, d, _ = ops.fused_classifier(wk["logits"], wk["tgt"], wk["V"])
+        act = ops.gelu_forward(y, "tanh")
+        return [y, mean, rstd, dx, dgamma, dbeta, dwte, dwpe, loss, row, d, act]
+
+    works = [work(500), work(600)]
+    alone = [run(w) for w in works]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=DEV), torch.cuda.Stream(device=DEV)]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    together = [None, None]
+    for rep in range(3):  # interleave the submissions
+        for k, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                together[k] = run(works[k])
+    torch.cuda.synchronize()
+    for k in range(2):
+        for i, (a, b) in enumerate(zip(alone[k], together[k])):
+            assert_bit_exact(b, a, f"stream {k} output {i}")
