@@ -857,6 +857,125 @@ def test_xl_adamw(ops, co):
     torch.cuda.empty_cache()
 
 
+# ------------------------------------------------ more than 2^31 elements per tensor
+# Element offsets past 2^31 (and byte offsets past 2^32) in every kernel family; the oracle runs
+# on slices taken from the start, the middle and the very end.
+BIG = 2**31 + 2**20 + 24
+
+
+def _gpu_randn(shape, seed, dtype, std=1.0):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    out = torch.empty(shape, dtype=dtype, device=DEV)
+    rows = shape[0]
+    step = max(1, rows // 8)
+    for r0 in range(0, rows, step):  # in pieces: the fp32 staging buffer stays small
+        piece = out[r0:r0 + step]
+        piece.copy_(torch.randn(piece.shape, generator=g, device=DEV) * std)
+    return out
+
+
+def test_big_gelu(ops, co):
+    x = _gpu_randn((BIG,), 1401, torch.bfloat16, 1.5)
+    dy = _gpu_randn((BIG,), 1402, torch.bfloat16)
+    y = ops.gelu_forward(x, "tanh")
+    dx = ops.gelu_backward(dy, x, "tanh")
+    for a in (0, 2**31 - 4096, BIG - 5000):
+        sl = slice(a, a + 5000)
+        assert_close(y[sl], co.gelu_forward(x[sl].cpu(), "tanh"), atol=1e-6, name=f"y[{a}:]")
+        assert_close(dx[sl], co.gelu_backward(dy[sl].cpu(), x[sl].cpu(), "tanh"), atol=1e-6, name=f"dx[{a}:]")
+    del x, dy, y, dx
+    torch.cuda.empty_cache()
+
+
+def test_big_layernorm(ops, co):
+    C = 1600
+    rows = BIG // C + 7
+    x = _gpu_randn((rows, C), 1403, torch.bfloat16)
+    dy = _gpu_randn((rows, C), 1404, torch.bfloat16)
+    gamma, beta = randn((C,), 1405, mean=1.0, std=0.02), randn((C,), 1406, std=0.02)
+    y, mean, rstd = ops.layernorm_forward(x, dev(gamma), dev(beta))
+    dx, dgamma, dbeta = ops.layernorm_backward(dy, x, mean, rstd, dev(gamma))
+    for a in (0, rows // 2, rows - 300):
+        sl = slice(a, a + 300)
+        y2, mean2, rstd2 = co.layernorm_forward(x[sl].cpu(), gamma, beta)
+        assert_close(y[sl], y2, atol=1e-6, name=f"y[{a}:]")
+        assert_close(mean[sl], mean2.flatten(), atol=1e-6, name=f"mean[{a}:]")
+        dx2, _, _ = co.layernorm_backward(dy[sl].cpu(), x[sl].cpu(), mean2, rstd2, gamma)
+        assert_close(dx[sl], dx2, atol=1e-6, name=f"dx[{a}:]")
+    # dbeta is the column sum of dy over all rows: ~N(0, rows), so the fp32 sum of `rows` terms is good
+    # to a few e-4 of its spread; torch's own column sum (fp32 tree over the same data) as the check
+    want = dy.float().sum(0)
+    assert (dbeta - want).abs().max().item() < 2e-3 * math.sqrt(rows)
+    del x, dy, y, dx
+    torch.cuda.empty_cache()
+
+
+def test_big_cross_entropy(ops, co):
+    V, stride = 50257, 50304
+    N = BIG // stride + 3
+    gx = _gpu_randn((N, stride), 1407, torch.bfloat16, 2.0)
+    t = randint(0, V, (N,), 1408)
+    t[5] = -100
+    pick = torch.tensor([0, 1, 5, N // 2, 2**31 // stride, 2**31 // stride + 1, N - 2, N - 1])
+    x_pick = gx[pick.to(DEV)].cpu()
+    loss, row, d, tw = ops.fused_classifier(gx, dev(t), V, inplace=True)
+    assert tw.item() == N - 1
+    assert abs(loss.item() - row.double().sum().item() / (N - 1)) < 1e-5
+    _, row2, d2, _ = co.cross_entropy(x_pick, t[pick], V, reduction="sum", dloss=1.0 / (N - 1))
+    assert_close(row[pick.to(DEV)], row2.float(), atol=1e-5, name="row loss sample")
+    assert_close(gx[pick.to(DEV)], d2, atol=1e-10, name="dlogits sample")
+    del gx
+    torch.cuda.empty_cache()
+
+
+def test_big_embedding(ops, co):
+    V, C = 50257, 1600
+    n = BIG // C + 5  # tokens
+    ids = randint(0, V, (n,), 1409)
+    w = _gpu_randn((V, C), 1410, torch.bfloat16, 0.02)
+    out = ops.embedding_forward(w, dev(ids))
+    w_cpu = w.cpu()
+    for a in (0, n // 2, n - 400):
+        sl = slice(a, a + 400)
+        assert_bit_exact(out[sl], co.embedding_forward(w_cpu, ids[sl]), f"rows {a}:")
+    # backward over the same number of tokens: every row of the table collects ~27 of them
+    dwte = ops.embedding_backward(out, dev(ids), V)
+    rows = torch.tensor([0, 17, V // 2, V - 1])
+    for r in rows.tolist():
+        hits = (ids == r).sum().item()
+        want = w_cpu[r].float() * hits  # out[i] == w[ids[i]], so row r of the gradient is hits * w[r]
+        assert_close(dwte[r].float().cpu(), want, atol=4e-4 * hits, name=f"dwte[{r}] ({hits} tokens)")  # one bf16 ulp at 0.1 * hits
+    del out, dwte, w
+    torch.cuda.empty_cache()
+
+
+def test_big_adamw(ops, co):
+    n = BIG
+    g = torch.Generator(device=DEV).manual_seed(1411)
+    w = torch.empty(n, device=DEV).normal_(0, 0.02, generator=g)
+    grad = torch.empty(n, device=DEV).normal_(0, 1e-3, generator=g)
+    m, v = torch.zeros(n, device=DEV), torch.zeros(n, device=DEV)
+    cuts = (0, 2**31 - 3000, n - 5000)
+    w0 = {a: w[a:a + 5000].cpu() for a in cuts}
+    ops.adamw_step(w, grad, m, v, t=1, **HYPER)
+    for a in cuts:
+        sl = slice(a, a + 5000)
+        ww, mm, vv, _ = co.adamw_step(w0[a], grad[sl].cpu(), torch.zeros(5000), torch.zeros(5000), t=1, **HYPER)
+        assert_close(w[sl], ww, atol=1e-8, name=f"w[{a}:]")
+        assert_close(m[sl], mm, atol=1e-10, name=f"m[{a}:]")
+        assert_close(v[sl], vv, atol=1e-13, name=f"v[{a}:]")
+    # one tensor of the multi-tensor launch past 2^31 elements as well
+    opt = ops.MultiTensorAdamW([w[:1000], w[1000:]], [grad[:1000], grad[1000:]], t=0, **HYPER)
+    w1 = {a: w[a:a + 5000].cpu() for a in cuts}
+    opt.step()
+    for a in cuts[1:]:
+        sl = slice(a, a + 5000)
+        ww, _, _, _ = co.adamw_step(w1[a], grad[sl].cpu(), torch.zeros(5000), torch.zeros(5000), t=1, **HYPER)
+        assert_close(w[sl], ww, atol=1e-8, name=f"multi w[{a}:]")
+    del opt, w, grad, m, v
+    torch.cuda.empty_cache()
+
+
 # ------------------------------------------------------------- empty inputs
 def test_empty_inputs(ops, co):
     """Zero rows / tokens / elements: every call returns without launching anything harmful and
