@@ -178,6 +178,84 @@ __device__ __forceinline__ void positions_vector(const T *__restrict__ dout, T *
   store16_stream(dwpe + f * VN, o);
 }
 
+// The same for a workgroup of kTile lanes, with the batch dimension split over S = 2^log2_s lanes
+// per vector: a lane walks its rows with 8 loads in flight, so a long batch is a long chain of
+// round trips unless it is cut up.  Lane (v, q) adds the rows of slice q for vector v of the
+// workgroup's kTile / S; slices 1.. are left in LDS and slice 0 adds them in order, so the sum
+// is a fixed tree.  lds: (S - 1) * (kTile / S) * VN floats.  With S = 1 this is positions_vector.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kPosMaxLog2Slices = 4;
+constexpr size_t kPosLdsBytes = (size_t)kTile * 32;  // bound for every S and element type
+
+template <typename T>
+__device__ __forceinline__ void positions_block(const T *__restrict__ dout, T *__restrict__ dwpe,
+                                                int64_t blk, int64_t B, int64_t TC, int accumulate,
+                                                int log2_s, f32x4 *lds, int tid) {
+  constexpr int VN = Vec16<T>::n;
+  constexpr int kPieces = VN / 4;  // f32x4 pieces of one vector's sums
+  if (log2_s == 0) {  // block-uniform
+    const int64_t f = blk * kTile + tid;
+    if (f < TC / VN) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
+    return;
+  }
+  constexpr int kInFlight = 4;  // loads per lane: with the batch cut up there are lanes enough
+  const int S = 1 << log2_s;
+  const int V = kTile >> log2_s;
+  const int v = tid & (V - 1);
+  const int q = tid >> (10 - log2_s);
+  static_assert(kTile == 1024, "q is tid / V with V = 1024 >> log2_s");
+  const int64_t f = blk * V + v;
+  const bool ok = f < TC / VN;
+  const int64_t per = (B + S - 1) / S;
+  const int64_t b_lo = q * per;
+  const int64_t b_hi = b_lo + per < B ? b_lo + per : B;
+  float a[VN];
+#pragma unroll
+  for (int k = 0; k < VN; ++k) a[k] = 0.f;
+  if (ok) {
+    for (int64_t b0 = b_lo; b0 < b_hi; b0 += kInFlight) {
+      Vec16<T> r[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u)
+        if (b0 + u < b_hi) r[u] = load16(dout + (b0 + u) * TC + f * VN);
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u)
+        if (b0 + u < b_hi)
+#pragma unroll
+          for (int k = 0; k < VN; ++k) a[k] += to_acc(r[u].e[k]);
+    }
+  }
+  if (q > 0 && ok) {
+#pragma unroll
+    for (int h = 0; h < kPieces; ++h) {
+      const f32x4 piece = {a[4 * h], a[4 * h + 1], a[4 * h + 2], a[4 * h + 3]};
+      lds[((q - 1) * kPieces + h) * V + v] = piece;
+    }
+  }
+  __syncthreads();
+  if (q != 0 || !ok) return;
+  for (int qq = 1; qq < S; ++qq) {
+#pragma unroll
+    for (int h = 0; h < kPieces; ++h) {
+      const f32x4 piece = lds[((qq - 1) * kPieces + h) * V + v];
+      a[4 * h] += piece.x;
+      a[4 * h + 1] += piece.y;
+      a[4 * h + 2] += piece.z;
+      a[4 * h + 3] += piece.w;
+    }
+  }
+  Vec16<T> o;
+  if (accumulate) {
+    const Vec16<T> old = load16(dwpe + f * VN);
+#pragma unroll
+    for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(to_acc(old.e[k]) + a[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(a[k]);
+  }
+  store16_stream(dwpe + f * VN, o);
+}
+
 // Zero fill of the table, spread over the sort and merge launches, whose own work leaves
 // most CUs idle.  Every row is zeroed before the reduce launch writes the indexed ones.
 // One fill workgroup clears kFillVecs 16-byte vectors.
@@ -208,8 +286,11 @@ __global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
     const IdxT *__restrict__ ids, KeyT *__restrict__ tiles, uint32_t *__restrict__ sorted_id,
     int64_t n, int n_tiles, int shift, int64_t num_weights, int64_t padding_idx,
     const T *__restrict__ dout, T *__restrict__ dwpe, int64_t B, int64_t TC, int accumulate,
-    int64_t pos_blocks, u32x4 *__restrict__ fill_dst, int64_t fill_vecs) {
-  __shared__ KeyT keys[2][kTile];
+    int64_t pos_blocks, int pos_log2_slices, u32x4 *__restrict__ fill_dst, int64_t fill_vecs) {
+  // the sorting workgroups keep two key arrays here, the position workgroups their slice sums
+  static_assert(2 * kTile * sizeof(KeyT) <= kPosLdsBytes, "the key arrays fit the shared buffer");
+  __shared__ f32x4 shared_raw[kPosLdsBytes / sizeof(f32x4)];
+  KeyT(*keys)[kTile] = reinterpret_cast<KeyT(*)[kTile]>(shared_raw);
   const int tid = threadIdx.x;
   const int64_t blk = blockIdx.x;
   if (blk > n_tiles + pos_blocks) {
@@ -217,8 +298,7 @@ __global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
     return;
   }
   if (blk > n_tiles) {
-    const int64_t f = (blk - n_tiles - 1) * kTile + tid;
-    if (f < TC / Vec16<T>::n) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
+    positions_block<T>(dout, dwpe, blk - n_tiles - 1, B, TC, accumulate, pos_log2_slices, shared_raw, tid);
     return;
   }
   if (blk == n_tiles) {
@@ -361,10 +441,10 @@ __global__ __launch_bounds__(kRankThreads) void emb_bwd_rank_kernel(
     const IdxT *__restrict__ ids, uint32_t *__restrict__ sorted_id,
     uint32_t *__restrict__ sorted_pos, int64_t n, int n_quads, int shift, int64_t num_weights,
     int64_t padding_idx, const T *__restrict__ dout, T *__restrict__ dwpe, int64_t B, int64_t TC,
-    int accumulate, int rank_blocks, int64_t pos_blocks, u32x4 *__restrict__ fill_dst,
-    int64_t fill_vecs) {
+    int accumulate, int rank_blocks, int64_t pos_blocks, int pos_log2_slices,
+    u32x4 *__restrict__ fill_dst, int64_t fill_vecs) {
   typedef KeyT Quad __attribute__((ext_vector_type(4)));
-  extern __shared__ u32x4 rank_lds[];
+  extern __shared__ u32x4 rank_lds[];  // the key list and the partial counts; kPosLdsBytes at least when positions are sliced
   __shared__ int valid_of_wave[kRankThreads / kWave];
   const int tid = threadIdx.x;
   const int64_t blk = blockIdx.x;
@@ -373,8 +453,8 @@ __global__ __launch_bounds__(kRankThreads) void emb_bwd_rank_kernel(
     return;
   }
   if (blk >= rank_blocks) {
-    const int64_t f = (blk - rank_blocks) * kRankThreads + tid;
-    if (f < TC / Vec16<T>::n) positions_vector<T>(dout, dwpe, f, B, TC, accumulate);
+    positions_block<T>(dout, dwpe, blk - rank_blocks, B, TC, accumulate, pos_log2_slices,
+                       reinterpret_cast<f32x4 *>(rank_lds), tid);
     return;
   }
   KeyT *keys = reinterpret_cast<KeyT *>(rank_lds);  // [4 n_quads], padded with sentinels
@@ -568,8 +648,7 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
         const int slot = e == kOwn - 1 ? 1 : 0;
         // four columns per 16-byte LDS word; word (j*H + h)*64 + lane holds columns
         // (lane + 64 j)*VN + 4h .. + 3, so the lanes of a wave write consecutive words
-        typedef float f32x4 __attribute__((ext_vector_type(4)));
-        constexpr int H = VN / 4;
+                constexpr int H = VN / 4;
         f32x4 *dst = reinterpret_cast<f32x4 *>(lds) + (wave * 2 + slot) * (kChunkCols / 4);
 #pragma unroll
         for (int j = 0; j < kVpl; ++j)
@@ -875,21 +954,27 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   KeyT *tiles = reinterpret_cast<KeyT *>(ws + L.off_tiles);
   uint32_t *sorted_id = reinterpret_cast<uint32_t *>(ws + L.off_sorted_id);
   uint32_t *sorted_pos = reinterpret_cast<uint32_t *>(ws + L.off_sorted_pos);
-  const int64_t pos_blocks = fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)kTile) : 0;
+  // lanes per vector of the position sum: enough that a lane walks at most ~16 rows of the batch
+  int pos_log2_slices = 0;
+  while (pos_log2_slices < kPosMaxLog2Slices && (B >> pos_log2_slices) > 16) ++pos_log2_slices;
+  const int64_t pos_blocks =
+      fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)(kTile >> pos_log2_slices)) : 0;
   const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecs);
   const int64_t n_quads = ceil_div(n, (int64_t)4);
   if ((size_t)n_quads * 4 * sizeof(KeyT) <= kRankMaxKeyBytes) {
     // a short list: one launch ranks every key against all others
-    static_assert(kRankThreads == kTile, "the position blocks cover kTile vectors each");
+    static_assert(kRankThreads == kTile, "positions_block assumes kTile lanes");
     const int64_t rank_blocks = ceil_div(n_quads * 4, (int64_t)kRankOwn);
     const int64_t blocks = rank_blocks + pos_blocks + fill_blocks;
     if (blocks == 0) return CS_OK;
-    const size_t lds = (size_t)n_quads * 4 * sizeof(KeyT) + kRankPartBytes;
+    size_t lds = (size_t)n_quads * 4 * sizeof(KeyT) + kRankPartBytes;
+    if (pos_blocks > 0 && pos_log2_slices > 0 && lds < kPosLdsBytes) lds = kPosLdsBytes;
+    static_assert(kPosLdsBytes <= kRankMaxKeyBytes + kRankPartBytes, "within the limit asked for");
     const int st = allow_rank_lds<KeyT, IdxT, T>(kRankMaxKeyBytes + kRankPartBytes);
     if (st != CS_OK) return st;
     emb_bwd_rank_kernel<KeyT, IdxT, T><<<dim3((unsigned)blocks), dim3(kRankThreads), lds, s>>>(
         (const IdxT *)ids, sorted_id, sorted_pos, n, (int)n_quads, L.shift, num_weights, padding_idx,
-        dout, dwpe, B, TC, accumulate, (int)rank_blocks, pos_blocks, fill_dst, fill_vecs);
+        dout, dwpe, B, TC, accumulate, (int)rank_blocks, pos_blocks, pos_log2_slices, fill_dst, fill_vecs);
     return launch_status();
   }
   // whole fill workgroups to the sort launch, the remainder to the merge launch
@@ -902,7 +987,7 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   if (blocks > 0x7fffffffLL || mblocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
   emb_bwd_tile_sort_kernel<KeyT, IdxT, T><<<dim3((unsigned)blocks), dim3(kTile), 0, s>>>(
       (const IdxT *)ids, tiles, sorted_id, n, (int)L.n_tiles, L.shift, num_weights, padding_idx,
-      dout, dwpe, B, TC, accumulate, pos_blocks, fill_dst, sort_fill_vecs);
+      dout, dwpe, B, TC, accumulate, pos_blocks, pos_log2_slices, fill_dst, sort_fill_vecs);
   int st = launch_status();
   if (st != CS_OK) return st;
   emb_bwd_merge_kernel<KeyT><<<dim3((unsigned)mblocks), dim3(kThreads), 0, s>>>(

@@ -572,6 +572,25 @@ def test_embedding_config1(ops, co, kind):
                  name="positions alone")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,T,C,V", [(17, 64, 64, 300), (40, 64, 128, 1000), (100, 32, 72, 50), (300, 16, 256, 5000),
+                                     (64, 128, 768, 50257), (37, 700, 64, 900)])
+def test_embedding_backward_fused_long_batches(ops, co, dtype, B, T, C, V):
+    """Batches long enough that the position-table sum splits them over 2 .. 16 lanes per
+    vector (also where the batch does not divide evenly), on the ranking path (B * T <= 8192)
+    and the tile-sort path."""
+    ids = randint(0, V, (B, T), 130)
+    dout = randn((B, T, C), 131, dtype=dtype)
+    atol = 1e-6 if dtype == torch.bfloat16 else 4e-5
+    dwte, dwpe = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_close(dwpe, co.embedding_backward_positions(dout), atol=atol, name="dwpe")
+    assert_close(dwte, co.embedding_backward(dout, ids, V), atol=atol, name="dwte")
+    again = ops.embedding_backward_fused(dev(dout), dev(ids), V)
+    assert_bit_exact(again[1], dwpe, "dwpe rerun")
+    ops.embedding_backward_fused(dev(dout), dev(ids), V, dwte=again[0], dwpe=again[1])
+    assert_close(again[1], co.embedding_backward_positions(dout, dwpe=dwpe.cpu()), atol=atol, name="dwpe +=")
+
+
 # ---------------------------------------------------------- Cross entropy
 @pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
