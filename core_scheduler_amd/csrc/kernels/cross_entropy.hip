@@ -691,6 +691,8 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
       ignore_index, reduction, dloss)
         if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
           CS_CE_STREAM(13, 4);  // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
+        } else if (nvec <= 1024 * 4) {
+          CS_CE_STREAM(4, VN);
         } else if (nvec <= 1024 * 7) {
           CS_CE_STREAM(7, VN);
         } else {

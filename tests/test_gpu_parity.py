@@ -611,7 +611,7 @@ def test_cross_entropy_reference_test_case(ops, co, reduction, dtype):
 @pytest.mark.parametrize("N,V,stride", [(64, 50257, 50304), (8, 50304, 50304), (33, 1000, 1024), (16, 4000, 4096),
                                         (5, 16385, 16392), (7, 100, 100), (3, 130000, 130048), (4, 77, 77),
                                         (40, 50257, 50257), (600, 1001, 1003), (3, 70001, 70001), (33, 1000, 1003),
-                                        (5, 3, 3), (9, 1, 1), (6, 13, 17)])
+                                        (5, 3, 3), (9, 1, 1), (6, 13, 17), (300, 32000, 32000), (260, 20000, 20008)])
 def test_cross_entropy_shapes(ops, co, dtype, N, V, stride):
     x = randn((N, stride), 111, std=2.0, dtype=dtype)
     t = randint(0, V, (N,), 112)
