@@ -43,32 +43,62 @@ __device__ __forceinline__ bool target_counts(int64_t t, int64_t V, int64_t igno
   return t != ignore_index && t >= 0 && t < V;
 }
 
+// Both one-workgroup kernels below keep kSmallInFlight loads per lane in flight: with one load
+// at a time a quarter of a million rows took 75 us each.
+constexpr int kSmallInFlight = 8;
+
 __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t *__restrict__ targets,
                                                         int64_t N, int64_t V,
                                                         int64_t ignore_index,
                                                         int *__restrict__ ws_count,
                                                         float *__restrict__ ws_weight) {
   __shared__ int scratch[16];
+  const int tid = threadIdx.x;
   int c = 0;
-  for (int64_t i = threadIdx.x; i < N; i += 1024) c += target_counts(targets[i], V, ignore_index);
+  for (int64_t i0 = tid; i0 < N; i0 += (int64_t)1024 * kSmallInFlight) {
+    int64_t t[kSmallInFlight];
+#pragma unroll
+    for (int u = 0; u < kSmallInFlight; ++u) {
+      const int64_t i = i0 + (int64_t)u * 1024;
+      t[u] = i < N ? targets[i] : ignore_index;
+    }
+#pragma unroll
+    for (int u = 0; u < kSmallInFlight; ++u) c += target_counts(t[u], V, ignore_index);
+  }
   c = block_reduce(c, SumOp{}, 0, scratch);
-  if (threadIdx.x == 0) {
+  if (tid == 0) {
     *ws_count = c;
     *ws_weight = (float)c;
   }
 }
 
-// Fixed-order sum of the row losses: thread t adds rows t, t+1024, ...; the
-// 1024 sub-sums are folded by the butterfly.  Independent of scheduling.
+// Fixed-order sum of the row losses: thread t adds rows t, t+1024, ... into kSmallInFlight
+// interleaved sums, which are then added in order; the 1024 sub-sums are folded by the
+// butterfly.  Independent of scheduling.
 __global__ __launch_bounds__(1024) void ce_reduce_kernel(const float *__restrict__ row_loss,
                                                          int64_t N, const int *__restrict__ ws_count,
                                                          int reduction, float *__restrict__ loss,
                                                          float *__restrict__ total_weight) {
   __shared__ float scratch[16];
+  const int tid = threadIdx.x;
+  float part[kSmallInFlight];
+#pragma unroll
+  for (int u = 0; u < kSmallInFlight; ++u) part[u] = 0.f;
+  for (int64_t i0 = tid; i0 < N; i0 += (int64_t)1024 * kSmallInFlight) {
+    float v[kSmallInFlight];
+#pragma unroll
+    for (int u = 0; u < kSmallInFlight; ++u) {
+      const int64_t i = i0 + (int64_t)u * 1024;
+      v[u] = i < N ? row_loss[i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kSmallInFlight; ++u) part[u] += v[u];
+  }
   float s = 0.f;
-  for (int64_t i = threadIdx.x; i < N; i += 1024) s += row_loss[i];
+#pragma unroll
+  for (int u = 0; u < kSmallInFlight; ++u) s += part[u];
   s = block_reduce(s, SumOp{}, 0.f, scratch);
-  if (threadIdx.x == 0) {
+  if (tid == 0) {
     const int c = *ws_count;
     if (loss) *loss = reduction == CS_REDUCTION_MEAN ? s / (float)c : s;
     if (total_weight) *total_weight = (float)c;
