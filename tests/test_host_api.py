@@ -381,6 +381,57 @@ def test_adamw_module_matches_torch_optimizer(host, sched):
 
 
 @pytest.mark.gpu
+def test_steps_without_host_waits_match_steps_with_waits(host, sched):
+    """The scheduler's stream rules are what keeps a step correct when nothing waits on the host:
+    gradients are produced on the assist stream (embedding backward) and on the main stream, the
+    optimizer reads both, zero_grad drops them, the next step starts at once.  Every kernel is
+    deterministic, so ten steps submitted back to back must give, bit for bit, the parameters of
+    the same ten steps with a host wait after every task."""
+    B, T, C, V = 4, 64, 256, 2000
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    first = None
+    results = []
+    for waits in (True, False, False):
+        root, mods = build_tree(host, sched, V=V, T=T, C=C)
+        if first is None:
+            first = {k: down(host, sched, p).clone() for k, p in root.named_parameters()}
+        for k, p in root.named_parameters():  # the same start for every run
+            host.assign_(sched, p, first[k].to(DEV))
+        opt = host.AdamWModule(sched, root, max_grad_norm=1.0, **hp)
+        gelu = host.GeLU.init(sched, 1)
+
+        def settle(*handles):
+            if waits:
+                for h in handles:
+                    h.wait()
+
+        # inputs are on the device before the first step, so no copy interrupts the submissions
+        inputs = [(randint(0, V, (B, T), 900 + step).to(DEV), randn((B, T, C), 950 + step).to(DEV)) for step in range(10)]
+        torch.cuda.synchronize()
+        for step in range(10):
+            ids = host.from_torch(sched, inputs[step][0])
+            x = mods["wte"].forward(sched, ids); settle(x)
+            y = mods["ln1"].forward(sched, x); settle(y)
+            a = host.GeLU.forward(sched, gelu, y); settle(a)
+            z = mods["lnf"].forward(sched, a); settle(z)
+            dz = host.from_torch(sched, inputs[step][1])  # upstream gradient of the step
+            da = mods["lnf"].backward(sched, dz); settle(da)
+            dy = host.GeLU.backward(sched, gelu, da); settle(dy)
+            dx = mods["ln1"].backward(sched, dy); settle(dx)
+            mods["wte"].backward(sched, dx)
+            opt.step(sched)
+            opt.zero_grad(sched)
+            if waits:
+                for _, p in root.named_parameters():
+                    p.wait()
+        results.append({k: down(host, sched, p) for k, p in root.named_parameters()})
+    for k in results[0]:
+        assert_bit_exact(results[1][k], results[0][k], f"{k}: no waits vs waits")
+        assert_bit_exact(results[2][k], results[0][k], f"{k}: no waits, again")
+    assert not torch.equal(results[0]["wte.weight"], first["wte.weight"])  # the steps did something
+
+
+@pytest.mark.gpu
 def test_clip_grad_norm_task_and_clipped_optimizer(host, sched, co):
     # Utils::clip_grad_norm_ (src/compute/utils.cpp:700-746) against torch.nn.utils.clip_grad_norm_,
     # then the module optimizer with max_grad_norm against clip + torch.optim.AdamW
