@@ -2,6 +2,12 @@
 // forward returns the loss; backward returns the gradient of the logits (no upstream gradient
 // argument: the reference feeds ones_like(loss)).  Here forward computes both in one pass and
 // keeps the gradient in state->backward.log_probs; backward hands it out.
+//
+// Logits are [N, columns] (two dimensions), targets [N] int64.  Rows whose target equals
+// ignore_index, or lies outside the class range, add nothing to the loss and get a zero
+// gradient; the mean is over the other rows.  label_smoothing other than 0 aborts in init, as
+// in the reference.  Inside the autocast guard the gradient of 16-bit logits is fp32 (what
+// ATen's autocast rule gives the reference); outside it keeps the logits' type.
 #pragma once
 #include <ATen/core/Reduction.h>
 
@@ -15,14 +21,14 @@ struct CS_API CrossEntropy {
     struct Forward {
       ReadOnlyTensor weight;  // per-class weights: never set by any caller of the reference
     } forward;
-    struct Backward {
-      ReadOnlyTensor total_weight;
-      ReadOnlyTensor log_probs;  // holds d(loss)/d(logits) after forward
+    struct Backward {  // filled by forward, released by backward
+      ReadOnlyTensor total_weight;  // number of rows that counted, as a 0-d fp32 tensor
+      ReadOnlyTensor log_probs;     // holds d(loss)/d(logits) after forward
       ReadOnlyTensor target;
       ReadOnlyTensor loss;
     } backward;
     struct Args {
-      int64_t reduction;
+      int64_t reduction;  // at::Reduction::{None, Mean, Sum}
       int64_t ignore_index;
       double label_smoothing;
       int64_t num_classes;  // class columns of the logits; < 0: all of them (the reference)

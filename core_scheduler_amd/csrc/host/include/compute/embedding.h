@@ -1,4 +1,13 @@
 // cs::compute::Embedding, the reference's op interface (include/compute/embedding.h:24-79).
+//
+// init draws the table from N(0, 1) ([num_embeddings, embedding_dim]), turns a negative
+// padding_idx into its row number and rejects max_norm, as the reference does.  forward
+// gathers rows for int32 or int64 indices of any shape (the result has the indices' shape
+// plus the embedding dimension) and keeps the indices.  backward runs on the assist stream
+// and leaves the dense gradient in state->forward.grad_weight: rows that were never indexed
+// are zero, the padding row gets nothing, and the sum over the tokens of a row is taken in a
+// fixed order (sort and segment, no floating point atomics), so two runs give the same bits.
+// A defined grad_weight is accumulated into, an undefined one assigned.
 #pragma once
 #include "arg.h"
 #include "module/state.h"
@@ -9,15 +18,15 @@ namespace cs::compute {
 struct CS_API Embedding {
   struct State : virtual module::State {
     struct Forward {
-      Tensor weight;
-      Tensor grad_weight{};
+      Tensor weight;         // [num_embeddings, embedding_dim]
+      Tensor grad_weight{};  // same shape; undefined until the first backward
     } forward;
     struct Backward {
-      ReadOnlyTensor indices;
+      ReadOnlyTensor indices;  // saved by forward, released by backward
     } backward;
     struct Args {
       int64_t num_weights;
-      int64_t padding_idx;
+      int64_t padding_idx;  // -1: none
       c10::optional<double> max_norm;
       double norm_type;
       bool scale_grad_by_freq;
@@ -25,7 +34,7 @@ struct CS_API Embedding {
     } args;
 
     State(const Forward &forward, const Backward &backward, const Args &args);
-    [[nodiscard]] OrderedDict<std::string, Tensor> parameters() const override;
+    [[nodiscard]] OrderedDict<std::string, Tensor> parameters() const override;  // "weight"
     [[nodiscard]] OrderedDict<std::string, Tensor> gradients() const override;
     [[nodiscard]] OrderedDict<std::string, Increment> increments() const override;
     void zero_grad() override;

@@ -1,4 +1,12 @@
 // cs::compute::LayerNorm, the reference's op interface (include/compute/layer_norm.h:24-87).
+//
+// init makes gamma = 1 and beta = 0 of `normalized_shape` (one trailing dimension here: the
+// kernels normalise rows of C = normalized_shape[0] columns).  forward writes y and keeps the
+// input and the per-row statistics for backward: mean and rstd = 1/sqrt(biased variance + eps),
+// fp32 whatever the input type.  backward returns dx and leaves dgamma / dbeta in
+// state->forward.grad_weight / grad_bias: assigned when those handles are undefined,
+// accumulated into otherwise.  Under the autocast guard y and dx are fp32 for 16-bit inputs,
+// as at::native_layer_norm behaves with fp32 parameters.
 #pragma once
 #include "arg.h"
 #include "module/state.h"
@@ -9,15 +17,15 @@ namespace cs::compute {
 struct CS_API LayerNorm {
   struct State : virtual module::State {
     struct Forward {
-      Tensor weight;
-      Tensor bias{};
-      Tensor grad_weight{};
-      Tensor grad_bias{};
+      Tensor weight;         // gamma [C]
+      Tensor bias{};         // beta [C]; stays an empty handle with Options::bias(false)
+      Tensor grad_weight{};  // dgamma, undefined until the first backward
+      Tensor grad_bias{};    // dbeta
     } forward;
-    struct Backward {
+    struct Backward {  // filled by forward, released once backward has been submitted
       ReadOnlyTensor input{};
-      ReadOnlyTensor mean{};
-      ReadOnlyTensor rstd{};
+      ReadOnlyTensor mean{};  // [rows] fp32
+      ReadOnlyTensor rstd{};  // [rows] fp32
     } backward;
     struct Args {
       const IntArray normalized_shape;
@@ -27,6 +35,7 @@ struct CS_API LayerNorm {
     } args;
 
     State(const Forward &forward, const Backward &backward, const Args &args);
+    // "weight" and, if there is one, "bias"
     [[nodiscard]] OrderedDict<std::string, Tensor> parameters() const override;
     [[nodiscard]] OrderedDict<std::string, Tensor> gradients() const override;
     [[nodiscard]] OrderedDict<std::string, Increment> increments() const override;

@@ -1,4 +1,9 @@
 // What a tensor handle points to (the reference's include/internal/tensor_impl.h:30-59).
+//
+// Three things travel with the device tensor: the lane (stream) whose task produced it, the
+// event recorded on that stream after the task, and the autocast request in force when the
+// handle was made.  A consumer on another lane makes its stream wait for the event unless the
+// event has completed already; a consumer on the same lane relies on stream order.
 #pragma once
 #include <ATen/core/TensorBody.h>
 
@@ -8,10 +13,13 @@
 
 namespace cs {
 struct ReadOnlyTensor::Impl {
+  // lane of the producing task; kNumPriority for tensors that came from outside (from_torch),
+  // which every consumer then waits for
   Task::Impl::Priority priority_ = Task::Impl::kMain;
   auto &priority() { return priority_; }
   auto &priority() const { return priority_; }
 
+  // recorded by the scheduler after the producing task's body has enqueued its kernels
   Event event_;
   auto &event() { return event_; }
   auto &event() const { return event_; }
@@ -28,6 +36,7 @@ struct ReadOnlyTensor::Impl {
   [[nodiscard]] auto sizes() const { return tensor_.sizes(); }
   [[nodiscard]] auto size(const int64_t dim) const { return tensor_.size(dim); }
   [[nodiscard]] auto numel() const { return tensor_.numel(); }
+  // task bodies assign here; undefined until the producing task has been submitted
   auto &tensor() { return tensor_; }
 
   at::Tensor tensor_{};

@@ -1,5 +1,12 @@
 // cs::module::Module: a tree of named submodules, each with at most one parameter state
 // (the reference's include/module/module.h:27-69, src/module/module.cpp:33-127).
+//
+// The tree exists to name things.  A leaf (Embedding, LayerNorm) registers the State of its
+// op; a container registers children under names without dots.  named_states() walks the tree
+// depth first in registration order and joins the names with '.', and named_parameters /
+// named_gradients / named_increments append the key the state uses for each tensor, which
+// gives the "h.0.ln_1.weight" names that checkpoints and optimizers go by.  Modules hold no
+// device memory of their own; zero_grad() and to() forward to the states.
 #pragma once
 #include <torch/nn/pimpl.h>
 
@@ -22,13 +29,17 @@ struct CS_API Module : std::enable_shared_from_this<Module> {
   // this module first (under `name_prefix`), then every submodule
   void apply(const ConstNamedModuleApplyFunction &function, const std::string &name_prefix = {}) const;
 
+  // at most one state per module: a second call replaces the first
   void register_state(std::shared_ptr<State> state);
 
+  // Adds a child and returns it.  Throws std::runtime_error for an empty name, a name with a
+  // dot in it or a name already taken.  The second form takes a holder (cs::module::LayerNorm).
   template <typename ModuleType>
   std::shared_ptr<ModuleType> register_module(std::string name, std::shared_ptr<ModuleType> module);
   template <typename ModuleType>
   std::shared_ptr<ModuleType> register_module(std::string name, torch::nn::ModuleHolder<ModuleType> module_holder);
 
+  // keys are module paths ("h.0.ln_1"); modules without a state do not appear
   OrderedDict<std::string, std::shared_ptr<State>> named_states() const;
   // keys are "<module path>.<name inside the state>", e.g. "wte.weight"
   OrderedDict<std::string, Tensor> named_parameters(bool recurse = true) const;
@@ -36,6 +47,7 @@ struct CS_API Module : std::enable_shared_from_this<Module> {
   OrderedDict<std::string, State::Increment> named_increments(bool recurse = true) const;
 
   void zero_grad() const;  // gradients become undefined handles
+  // converts every parameter (dtype / device of `options`); gradients are dropped
   void to(TensorOptions options) const;
 
  protected:

@@ -1,4 +1,12 @@
 // Parameter / gradient bookkeeping interfaces (the reference's include/module/state.h:36-52).
+//
+// An op that owns parameters (Embedding, LayerNorm) derives its State from module::State and
+// names what it holds: parameters() and gradients() use the same keys ("weight", "bias"), and
+// increments() pairs each parameter with its gradient, which is what an optimizer walks.
+// A gradient handle is undefined until a backward task has produced it; the first backward
+// after zero_grad() assigns (`=`), later ones accumulate (`+=`).  zero_grad() makes the handles
+// undefined again rather than filling them with zeros, as the reference does
+// (src/compute/embedding.cpp:54, src/compute/layer_norm.cpp:69-74).
 #pragma once
 #include <torch/ordered_dict.h>
 
@@ -12,6 +20,7 @@ using OrderedDict = torch::OrderedDict<Key, Value>;
 }
 
 namespace cs::module {
+// What an optimizer keeps per parameter (moments, step count, hyper-parameters).
 struct OptimizerState {
   virtual ~OptimizerState() = default;
   virtual void set_lr(double lr) const = 0;
@@ -21,7 +30,7 @@ struct OptimizerState {
 struct CS_API State {
   struct Increment {
     Tensor parameter;
-    Tensor gradient;
+    Tensor gradient;  // undefined: the parameter took no part in the last backward pass
   };
   virtual ~State() = default;
   [[nodiscard]] virtual OrderedDict<std::string, Tensor> parameters() const = 0;
