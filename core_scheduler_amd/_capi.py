@@ -20,6 +20,7 @@ GELU_ERF, GELU_TANH = 0, 1
 
 OK = 0
 ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_MISALIGNED, ERR_WORKSPACE, ERR_TOO_LARGE = -1, -2, -3, -4, -5
+ERR_STATIC_LIMIT = -6
 
 
 class AdamWTensor(ctypes.Structure):
@@ -104,6 +105,11 @@ SIGNATURES = {
     "cs_fused_classifier": (
         c_int,
         [c_void_p] * 7 + [c_size_t] + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_void_p],
+    ),
+    "cs_fused_classifier_static_max_rows": (c_int64, []),
+    "cs_fused_classifier_static": (
+        c_int,
+        [c_void_p] * 6 + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_void_p],
     ),
     "cs_fused_classifier_phases": (
         c_int,

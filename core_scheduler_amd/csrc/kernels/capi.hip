@@ -44,6 +44,8 @@ extern "C" const char *cs_hip_error_string(int code) {
     case CS_ERR_MISALIGNED: return "pointer not aligned to its element size";
     case CS_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case CS_ERR_TOO_LARGE: return "size beyond what one launch can address";
+    case CS_ERR_STATIC_LIMIT:
+      return "size beyond the library's built-in scratch buffer; use the entry point that takes a workspace";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

@@ -869,6 +869,57 @@ extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int6
   return ce_run(a, 1 | 2 | 4, stream);
 }
 
+// ------------------------------------------------- the call that allocates nothing
+// Device memory that belongs to the library, one copy per GPU, held until the process ends:
+// the workspace of cs_fused_classifier_static.  In host code this name is only a handle for
+// hipGetSymbolAddress; the address that kernels and the host use is the one that call returns.
+static __device__ __align__(256) unsigned char scratch[CS_FUSED_CLASSIFIER_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+// the scratch array's address on each device, looked up once per device (threads may race to
+// fill a slot: they store the same value)
+std::atomic<void *> scratch_ptr[kMaxDevices];
+
+int static_scratch(void **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return CS_ERR_UNSUPPORTED;
+  void *p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    // the current device's copy of the array
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return CS_ERR_WORKSPACE;
+    scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return CS_OK;
+}
+}  // namespace
+
+extern "C" int64_t cs_fused_classifier_static_max_rows(void) {
+  return ((int64_t)CS_FUSED_CLASSIFIER_STATIC_SCRATCH_BYTES - (int64_t)kWsHeader) / (int64_t)sizeof(float);
+}
+
+extern "C" int cs_fused_classifier_static(const void *logits, void *dlogits, const int64_t *targets,
+                                          float *row_loss, float *loss, float *total_weight,
+                                          int64_t N, int64_t V, int64_t row_stride,
+                                          int64_t ignore_index, int reduction, float dloss,
+                                          int dtype, int dlogits_dtype, void *stream) {
+  if (N > cs_fused_classifier_static_max_rows()) return CS_ERR_STATIC_LIMIT;
+  void *ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != CS_OK) return st;
+  // Nothing in the scratch has to start at zero: the counting launch overwrites the header and
+  // the row pass overwrites the N row losses that the reduction then reads.
+  const CeArgs a{logits, dlogits, targets, row_loss, loss, total_weight, ws,
+                 (size_t)CS_FUSED_CLASSIFIER_STATIC_SCRATCH_BYTES, N, V, row_stride, ignore_index,
+                 reduction, dloss, dtype, dlogits_dtype};
+  return ce_run(a, 1 | 2 | 4, stream);
+}
+
 extern "C" int cs_fused_classifier_phases(const void *logits, void *dlogits,
                                           const int64_t *targets, float *row_loss, float *loss,
                                           float *total_weight, void *workspace,

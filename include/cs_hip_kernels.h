@@ -68,6 +68,8 @@ enum cs_error {
   CS_ERR_MISALIGNED = -3,       /* pointer not aligned to its element size  */
   CS_ERR_WORKSPACE = -4,        /* workspace missing or too small           */
   CS_ERR_TOO_LARGE = -5,        /* size beyond what the launch can address  */
+  CS_ERR_STATIC_LIMIT = -6,     /* size beyond the library's built-in scratch:
+                                   use the entry point that takes a workspace */
 };
 
 int cs_hip_abi_version(void);
@@ -329,6 +331,30 @@ int cs_fused_classifier_phases(const void *logits, void *dlogits,
                                int64_t ignore_index, int reduction,
                                float dloss, int dtype, int dlogits_dtype,
                                int phases, void *stream);
+
+/* cs_fused_classifier for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): the same launches and the same results, with the workspace
+ * taken from an array of CS_FUSED_CLASSIFIER_STATIC_SCRATCH_BYTES that the
+ * library itself holds in device memory on every GPU it runs on, until the
+ * process ends.  It has no counterpart in the reference.  It allocates
+ * nothing and frees nothing, on the device or through any library.
+ * Limit: N <= cs_fused_classifier_static_max_rows() (262,080 rows for the
+ * 1 MiB array); more rows return CS_ERR_STATIC_LIMIT and launch nothing.
+ * All calls on one GPU share that GPU's array, which keeps what the last
+ * call left there (no call needs it cleared): calls that overlap on one GPU,
+ * on different streams or from different threads, race on it and must be
+ * ordered by the caller.  The first call on a device looks up the array's
+ * address on that device (hipGetSymbolAddress), later calls reuse it. */
+#define CS_FUSED_CLASSIFIER_STATIC_SCRATCH_BYTES (1 << 20)
+int64_t cs_fused_classifier_static_max_rows(void);
+int cs_fused_classifier_static(const void *logits, void *dlogits,
+                               const int64_t *targets, float *row_loss,
+                               float *loss, float *total_weight, int64_t N,
+                               int64_t V, int64_t row_stride,
+                               int64_t ignore_index, int reduction,
+                               float dloss, int dtype, int dlogits_dtype,
+                               void *stream);
 
 #ifdef __cplusplus
 }

@@ -45,7 +45,7 @@ def test_binding_covers_the_header_exactly():
 def test_error_strings():
     lib = _capi.load()
     assert lib.cs_hip_error_string(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6):
         assert len(lib.cs_hip_error_string(code)) > 4
 
 
@@ -116,3 +116,13 @@ def test_ops_refuse_cpu_tensors():
 
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.gelu_forward(torch.zeros(8))
+
+
+def test_static_scratch_entry_point_rejects_sizes_beyond_its_array():
+    lib = _capi.load()
+    limit = lib.cs_fused_classifier_static_max_rows()
+    assert limit == ((1 << 20) - 256) // 4
+    p = ctypes.c_void_p(4096)  # never dereferenced: rejected before the HIP runtime is touched
+    code = lib.cs_fused_classifier_static(p, p, p, None, p, None, limit + 1, 8, 8, -100, _capi.REDUCTION_MEAN, 1.0,
+                                          _capi.F32, _capi.F32, None)
+    assert code == _capi.ERR_STATIC_LIMIT
