@@ -44,42 +44,81 @@ namespace {
 constexpr int kThreads = 256;
 
 // ------------------------------------------------------------------ forward
-// One 16-byte vector per thread step; `nvec` vectors per row.
+// One 16-byte vector per thread step, kFwdUnroll steps per thread; `nvec` vectors per row.
+// The row and the vector of a thread's first step come from one 32-bit division, the later
+// steps advance them by the constant 256 = step_rows * nvec + step_vecs.  Every load of a full
+// workgroup is issued without a lane-dependent condition (an index out of range reads row 0 and
+// the result is replaced by zeros): the position rows and the indices go first, the table rows
+// as soon as the indices are there, so a thread makes two round trips however many steps it has.
+#ifndef CS_EMB_FWD_UNROLL
+#define CS_EMB_FWD_UNROLL 2
+#endif
+constexpr int kFwdUnroll = CS_EMB_FWD_UNROLL;
+
 template <typename T, typename IdxT, bool ADD>
 __global__ __launch_bounds__(kThreads) void emb_fwd_vec_kernel(
     const T *__restrict__ weight, const T *__restrict__ wpe, const IdxT *__restrict__ ids,
-    T *__restrict__ out, int64_t n_rows, int nvec, int64_t num_weights, int64_t T_len) {
+    T *__restrict__ out, int64_t n_rows, uint32_t nvec, int64_t num_weights, uint32_t T_len) {
   constexpr int VN = Vec16<T>::n;
-  constexpr int kUnroll = 4;
+  constexpr uint32_t kChunk = kThreads * kFwdUnroll;
   const int64_t total = n_rows * nvec;
-  // one 64-bit division per workgroup, 32-bit ones per vector
-  const int64_t chunk_base = (int64_t)blockIdx.x * (kThreads * kUnroll);
-  const int64_t row_base = chunk_base / nvec;
-  const uint32_t rem_base = (uint32_t)(chunk_base - row_base * nvec);
-  const int64_t base = chunk_base + threadIdx.x;
-  Vec16<T> w[kUnroll], p[kUnroll];
-  bool ok[kUnroll];
+  // the workgroup's first row: 32-bit divisions where the whole output has fewer than 2^32
+  // vectors (a 64-bit division by a variable is a hundred instructions)
+  const int64_t chunk_base = (int64_t)blockIdx.x * kChunk;
+  int64_t row_base;
+  uint32_t rem_base, t_base = 0u;
+  if (total <= 0xFFFFFFFFll) {
+    const uint32_t cb = (uint32_t)chunk_base;
+    const uint32_t rb = cb / nvec;
+    rem_base = cb - rb * nvec;
+    if constexpr (ADD) t_base = rb % T_len;
+    row_base = rb;
+  } else {
+    row_base = chunk_base / nvec;
+    rem_base = (uint32_t)(chunk_base - row_base * nvec);
+    if constexpr (ADD) t_base = (uint32_t)(row_base % T_len);
+  }
+  const uint32_t step_rows = kThreads / nvec, step_vecs = kThreads % nvec;
+  const uint32_t local = rem_base + threadIdx.x;
+  uint32_t drow = local / nvec;
+  uint32_t vec = local - drow * nvec;
+  const bool full = chunk_base + kChunk <= total;  // workgroup-uniform
+
+  uint32_t drows[kFwdUnroll], vecs[kFwdUnroll];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const int64_t f = base + (int64_t)u * kThreads;
-    const uint32_t local = rem_base + (uint32_t)(u * kThreads) + threadIdx.x;
-    const int64_t row = row_base + local / (uint32_t)nvec;
-    const uint32_t vec = local % (uint32_t)nvec;
-    ok[u] = false;
-    if (f < total) {
-      const int64_t id = (int64_t)ids[row];
-      ok[u] = id >= 0 && id < num_weights;
-      if (ok[u]) w[u] = load16(weight + id * ((int64_t)nvec * VN) + (int64_t)vec * VN);
-      if constexpr (ADD) {
-        const int64_t t = row % T_len;
-        p[u] = load16(wpe + t * ((int64_t)nvec * VN) + (int64_t)vec * VN);
-      }
+  for (int u = 0; u < kFwdUnroll; ++u) {
+    drows[u] = drow;
+    vecs[u] = vec;
+    drow += step_rows;
+    vec += step_vecs;
+    if (vec >= nvec) {
+      vec -= nvec;
+      ++drow;
     }
   }
+  const int64_t row_stride = (int64_t)nvec * VN;
+  if (full) {
+    IdxT raw_id[kFwdUnroll];
+    Vec16<T> w[kFwdUnroll], p[kFwdUnroll];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const int64_t f = base + (int64_t)u * kThreads;
-    if (f < total) {
+    for (int u = 0; u < kFwdUnroll; ++u) raw_id[u] = ids[row_base + drows[u]];
+    if constexpr (ADD) {
+#pragma unroll
+      for (int u = 0; u < kFwdUnroll; ++u) {
+        uint32_t t = t_base + drows[u];  // below 2 T_len + 256: the workgroup spans few rows
+        t = t % T_len;
+        p[u] = load16(wpe + (int64_t)t * row_stride + (int64_t)vecs[u] * VN);
+      }
+    }
+    bool ok[kFwdUnroll];
+#pragma unroll
+    for (int u = 0; u < kFwdUnroll; ++u) {
+      const int64_t id = (int64_t)raw_id[u];
+      ok[u] = id >= 0 && id < num_weights;
+      w[u] = load16(weight + (ok[u] ? id : 0) * row_stride + (int64_t)vecs[u] * VN);
+    }
+#pragma unroll
+    for (int u = 0; u < kFwdUnroll; ++u) {
       Vec16<T> r;
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
@@ -90,8 +129,28 @@ __global__ __launch_bounds__(kThreads) void emb_fwd_vec_kernel(
           r.e[k] = ok[u] ? w[u].e[k] : T{};
         }
       }
-      store16_stream(out + f * VN, r);
+      store16_stream(out + ((row_base + drows[u]) * nvec + vecs[u]) * VN, r);
     }
+    return;
+  }
+  // the last, ragged workgroup
+  for (int u = 0; u < kFwdUnroll; ++u) {
+    const int64_t row = row_base + drows[u];
+    if (row >= n_rows) break;
+    const int64_t id = (int64_t)ids[row];
+    const bool ok = id >= 0 && id < num_weights;
+    Vec16<T> r;
+#pragma unroll
+    for (int k = 0; k < VN; ++k) r.e[k] = T{};
+    if (ok) {
+      r = load16(weight + id * row_stride + (int64_t)vecs[u] * VN);
+      if constexpr (ADD) {
+        const Vec16<T> pv = load16(wpe + (row % T_len) * row_stride + (int64_t)vecs[u] * VN);
+#pragma unroll
+        for (int k = 0; k < VN; ++k) r.e[k] = from_acc<T>(to_acc(r.e[k]) + to_acc(pv.e[k]));
+      }
+    }
+    store16_stream(out + (row * nvec + vecs[u]) * VN, r);
   }
 }
 
@@ -155,11 +214,15 @@ __device__ __forceinline__ void positions_vector(const T *__restrict__ dout, T *
   float a[VN];
 #pragma unroll
   for (int k = 0; k < VN; ++k) a[k] = 0.f;
+  // eight loads in flight, none under a condition (a batch row past the end re-reads the last
+  // one and is not added)
   for (int64_t b0 = 0; b0 < B; b0 += 8) {
     Vec16<T> v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (b0 + u < B) v[u] = load16(dout + (b0 + u) * TC + f * VN);
+    for (int u = 0; u < 8; ++u) {
+      const int64_t b = b0 + u < B ? b0 + u : B - 1;
+      v[u] = load16_stream(dout + b * TC + f * VN);
+    }
 #pragma unroll
     for (int u = 0; u < 8; ++u)
       if (b0 + u < B)
@@ -216,8 +279,10 @@ __device__ __forceinline__ void positions_block(const T *__restrict__ dout, T *_
     for (int64_t b0 = b_lo; b0 < b_hi; b0 += kInFlight) {
       Vec16<T> r[kInFlight];
 #pragma unroll
-      for (int u = 0; u < kInFlight; ++u)
-        if (b0 + u < b_hi) r[u] = load16(dout + (b0 + u) * TC + f * VN);
+      for (int u = 0; u < kInFlight; ++u) {
+        const int64_t b = b0 + u < b_hi ? b0 + u : b_hi - 1;
+        r[u] = load16_stream(dout + b * TC + f * VN);
+      }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u)
         if (b0 + u < b_hi)
@@ -259,7 +324,10 @@ __device__ __forceinline__ void positions_block(const T *__restrict__ dout, T *_
 // Zero fill of the table, spread over the sort and merge launches, whose own work leaves
 // most CUs idle.  Every row is zeroed before the reduce launch writes the indexed ones.
 // One fill workgroup clears kFillVecs 16-byte vectors.
-constexpr int kFillVecs = 8192;  // 128 KB
+#ifndef CS_EMB_FILL_VECS
+#define CS_EMB_FILL_VECS 2048
+#endif
+constexpr int kFillVecs = CS_EMB_FILL_VECS;  // 32 KB: 64 -> 61.6 us at 16384 tokens x 1600 against 128 KB pieces
 #ifndef CS_EMB_FILL_SORT_PCT
 #define CS_EMB_FILL_SORT_PCT 40  // share of the table cleared in the sort launch
 #endif
@@ -370,7 +438,7 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
 #pragma unroll
     for (int u = 0; u < kVecPerThread; ++u) {
       const int i = u * kThreads + threadIdx.x;
-      if (i < c_vecs) v[u] = src[i];
+      v[u] = src[i < c_vecs ? i : c_vecs - 1];  // all requested before the first is used
     }
     __syncthreads();  // the previous chunk is no longer being searched
 #pragma unroll
@@ -465,15 +533,25 @@ __global__ __launch_bounds__(kRankThreads) void emb_bwd_rank_kernel(
 
   // ---- every key of the list, and how many are real
   int mine = 0;
-  for (int i = tid; i < n_keys; i += kRankThreads) {
-    KeyT key = KeyCodec<KeyT>::kSentinel;
-    if (i < n) {
-      const int64_t id = (int64_t)ids[i];
-      if (id >= 0 && id < num_weights && id != padding_idx)
-        key = KeyCodec<KeyT>::make((uint32_t)id, (uint32_t)i, shift);
+  constexpr int kIdsInFlight = 8;  // the whole list of 8192 in one round trip
+  for (int i0 = tid; i0 < n_keys; i0 += kRankThreads * kIdsInFlight) {
+    IdxT raw[kIdsInFlight];
+#pragma unroll
+    for (int u = 0; u < kIdsInFlight; ++u) {
+      const int i = i0 + u * kRankThreads;
+      raw[u] = ids[i < n ? i : n - 1];  // no load under a condition: they all go out at once
     }
-    keys[i] = key;
-    mine += key != KeyCodec<KeyT>::kSentinel ? 1 : 0;
+#pragma unroll
+    for (int u = 0; u < kIdsInFlight; ++u) {
+      const int i = i0 + u * kRankThreads;
+      if (i >= n_keys) break;
+      KeyT key = KeyCodec<KeyT>::kSentinel;
+      const int64_t id = (int64_t)raw[u];
+      if (i < n && id >= 0 && id < num_weights && id != padding_idx)
+        key = KeyCodec<KeyT>::make((uint32_t)id, (uint32_t)i, shift);
+      keys[i] = key;
+      mine += key != KeyCodec<KeyT>::kSentinel ? 1 : 0;
+    }
   }
   const int in_wave = wave_reduce(mine, SumOp{});
   if (lane == 0) valid_of_wave[wave] = in_wave;
@@ -521,7 +599,10 @@ constexpr int kRedWaves = kWindow / kOwn;       // 8
 constexpr int kRedThreads = kRedWaves * kWave;  // 512: two workgroups share a CU
 constexpr int kFinThreads = 1024;               // finish kernel
 constexpr int kFinWaves = kFinThreads / kWave;
-constexpr int kVpl = 2;                         // 16-byte column vectors per lane per column chunk
+#ifndef CS_EMB_VPL
+#define CS_EMB_VPL 2
+#endif
+constexpr int kVpl = CS_EMB_VPL;                // 16-byte column vectors per lane per column chunk
 
 // Workgroup w reduces sorted entries [kWindow w, kWindow (w + 1)).  partial rows live at
 // partial[(w*2 + slot) * C]: slot 0 for a run that came in over the window's
@@ -546,17 +627,27 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
   const bool in_window = lane < kWindow;
   // lanes 0..3: the positions of this wave's four entries, asked for together with the ids
   // (an entry past the real ones holds no position; it is never used)
+  // The four index loads go out together: none sits under a lane-dependent condition (an entry
+  // past the end re-reads the last one and is masked afterwards).
   const int64_t own_p = p0 + wave * kOwn + lane;
-  const uint32_t lane_pos = (lane < kOwn && own_p < n) ? sorted_pos[own_p] : 0u;
-  const uint32_t my_id = (in_window && p < n) ? sorted_id[p] : kNoId;
-  const uint32_t prev_id = (in_window && p > 0 && p <= n) ? sorted_id[p - 1] : kNoId;
+  const int64_t last = n - 1;
+  const uint32_t raw_pos = sorted_pos[own_p < last ? own_p : last];
+  const uint32_t raw_id = sorted_id[p < last ? p : last];
+  const uint32_t raw_prev = sorted_id[p > 0 ? (p - 1 < last ? p - 1 : last) : 0];
+  uint32_t raw_next = sorted_id[p0 + kWindow < last ? p0 + kWindow : last];  // uniform load
+  // keeps the compiler from moving three of the loads below the early exit, where each would
+  // wait for the one before it
+  asm volatile("" : "+v"(raw_next) : "v"(raw_pos), "v"(raw_id), "v"(raw_prev));
+  const uint32_t lane_pos = (lane < kOwn && own_p < n) ? raw_pos : 0u;
+  const uint32_t my_id = (in_window && p < n) ? raw_id : kNoId;
+  const uint32_t prev_id = (in_window && p > 0 && p <= n) ? raw_prev : kNoId;
   const uint64_t valid = __ballot(my_id != kNoId);
   if (valid == 0) return;  // nothing sorted into this window
   const int n_valid = __popcll(valid);  // valid entries are a prefix of the window
   // true segment heads, and run starts inside the window (a head, or entry 0)
   const uint64_t heads = __ballot(my_id != kNoId && (p == 0 || my_id != prev_id));
   const uint64_t starts = heads | 1ull;
-  const uint32_t next_id = (p0 + kWindow < n) ? sorted_id[p0 + kWindow] : kNoId;  // uniform load
+  const uint32_t next_id = (p0 + kWindow < n) ? raw_next : kNoId;
   const uint32_t last_id = __shfl(my_id, n_valid - 1, kWave);
   const bool leaves = n_valid == kWindow && next_id == last_id;    // last run goes over the right edge
 
@@ -571,16 +662,16 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
   for (int cb = 0; cb < nvec; cb += kWave * kVpl) {
     // ---- level 1: this wave's four entries
     const int e0 = wave * kOwn;
+    // all kOwn * kVpl row loads are in flight before the first is used: an entry past the valid
+    // ones reads row 0, a vector past the row re-reads the row's last one; neither is added
     Vec16<T> r[kOwn][kVpl];
 #pragma unroll
     for (int e = 0; e < kOwn; ++e) {
-      if (e0 + e < n_valid) {
-        const int64_t pos = __shfl(lane_pos, e, kWave);
+      const int64_t pos = e0 + e < n_valid ? (int64_t)__shfl(lane_pos, e, kWave) : 0;
 #pragma unroll
-        for (int j = 0; j < kVpl; ++j) {
-          const int idx = cb + lane + kWave * j;
-          if (idx < nvec) r[e][j] = load16_stream(dout + pos * C + (int64_t)idx * VN);
-        }
+      for (int j = 0; j < kVpl; ++j) {
+        const int idx = cb + lane + kWave * j;
+        r[e][j] = load16_stream(dout + pos * C + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
       }
     }
     float acc[kVpl][VN];
@@ -872,11 +963,11 @@ int fwd_launch(const void *weight, const void *wpe, const void *ids, void *out, 
                       (!ADD || is_aligned16(wpe)) && C / VN <= 0x7fffffff;
   if (vec_ok) {
     const int64_t total = n_rows * (C / VN);
-    const int64_t blocks = ceil_div(total, (int64_t)kThreads * 4);
+    const int64_t blocks = ceil_div(total, (int64_t)kThreads * kFwdUnroll);
     if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
     emb_fwd_vec_kernel<T, IdxT, ADD><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-        (const T *)weight, (const T *)wpe, (const IdxT *)ids, (T *)out, n_rows, (int)(C / VN),
-        num_weights, T_len);
+        (const T *)weight, (const T *)wpe, (const IdxT *)ids, (T *)out, n_rows, (uint32_t)(C / VN),
+        num_weights, (uint32_t)T_len);
   } else {
     int64_t blocks = ceil_div(n_rows * C, (int64_t)kThreads);
     if (blocks > 65536) blocks = 65536;

@@ -82,6 +82,15 @@ const char *cs_hip_error_string(int code);
  * and the scale of the hardware traffic counters). */
 int cs_stream_copy(void *dst, const void *src, int64_t bytes, void *stream);
 
+/* The two halves of that calibration, also without counterpart in the
+ * reference: a read-only pass (every workgroup leaves one 32-bit word, the xor
+ * of what it read, in out[0 .. cs_stream_read_out_words(bytes))) and a
+ * write-only pass (dst filled with `value`).  Same rules for bytes and
+ * alignment as cs_stream_copy. */
+int64_t cs_stream_read_out_words(int64_t bytes);
+int cs_stream_read(const void *src, void *out, int64_t bytes, void *stream);
+int cs_stream_fill(void *dst, int64_t bytes, uint32_t value, void *stream);
+
 /* ------------------------------------------------------------------------
  * AdamW
  * replaces stepKernel / stepKernelAmsgrad and the step<UpT,T> kernels,

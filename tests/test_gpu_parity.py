@@ -1033,3 +1033,37 @@ def test_empty_inputs(ops, co):
     assert loss.item() == 0 and tw.item() == 0 and d.shape == (0, 128)
     loss, _, _, _ = ops.fused_classifier(x, t, 100)
     assert math.isnan(loss.item())
+
+
+# ------------------------------------------------------------ calibration kernels
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbytes", [16, 4096 * 3 + 16, (64 << 20) + 48])
+def test_stream_copy_read_fill(nbytes):
+    """The benchmark's calibration kernels move exactly the bytes they are asked to."""
+    import ctypes
+
+    from core_scheduler_amd import _capi
+
+    lib = _capi.load()
+    dev = torch.device("cuda:0")
+    P = ctypes.c_void_p
+    st = P(torch.cuda.current_stream(dev).cuda_stream)
+    g = torch.Generator(device="cpu").manual_seed(nbytes)
+    src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g).to(dev)
+    dst = torch.zeros(nbytes + 64, dtype=torch.uint8, device=dev)
+    _capi.check("cs_stream_copy", lib.cs_stream_copy(P(dst.data_ptr()), P(src.data_ptr()), nbytes, st))
+    assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
+    words = lib.cs_stream_read_out_words(nbytes)
+    out = torch.zeros(words, dtype=torch.int32, device=dev)
+    _capi.check("cs_stream_read", lib.cs_stream_read(P(src.data_ptr()), P(out.data_ptr()), nbytes, st))
+    want = 0
+    for w in src.cpu().numpy().view("<u4").tolist():
+        want ^= w
+    got = 0
+    for w in out.cpu().numpy().view("<u4").tolist():
+        got ^= w
+    assert got == want, "the read pass saw other bytes than the buffer holds"
+    _capi.check("cs_stream_fill", lib.cs_stream_fill(P(dst.data_ptr()), nbytes, 0x01020304, st))
+    torch.cuda.synchronize()
+    assert int(dst[nbytes:].sum()) == 0
+    assert bool((dst[:nbytes].view(torch.int32) == 0x01020304).all())
