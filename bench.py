@@ -59,7 +59,7 @@ def gpt2_param_sizes(n_layer, C, V=50257, T=1024):
 _BLOCKER = {}
 
 
-def hold_gpu(torch, ms=3.0):
+def hold_gpu(torch, ms=6.0):
     """Queues ~`ms` of plain copies so that the launches that follow are all enqueued while the
     GPU is still busy: the timed calls then run back to back, as they do inside a training step,
     instead of each waiting for the host to issue it."""
@@ -80,8 +80,21 @@ def _capi_lib():
     return _capi.load()
 
 
-def event_ms(fn, reps, torch):
-    """Median / mean duration of one call, each bracketed by its own pair of events."""
+def event_ms(fn, reps, torch, rounds=3):
+    """Duration of one call when `reps` calls run back to back: one pair of events around the
+    whole batch (no event, hence no gap, between the calls), median over `rounds` batches.  Also
+    returns the median of per-call event pairs, which carries the events' own cost (~3 us)."""
+    batch = []
+    for _ in range(rounds):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        hold_gpu(torch)
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        batch.append(e0.elapsed_time(e1) / reps)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
     torch.cuda.synchronize()
@@ -91,8 +104,8 @@ def event_ms(fn, reps, torch):
         fn(i)
         ends[i].record()
     torch.cuda.synchronize()
-    ts = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return statistics.median(ts), sum(ts) / len(ts)
+    per_call = statistics.median(s.elapsed_time(e) for s, e in zip(starts, ends))
+    return statistics.median(batch), per_call
 
 
 def run_headline(args, torch, ops, capi):
@@ -171,6 +184,12 @@ def per_op_table(args, torch, ops):
     def stream_copy(dst, src):
         lib.cs_stream_copy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), src.numel(), stream)
 
+    def stream_read(src, out):
+        lib.cs_stream_read(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(out.data_ptr()), src.numel(), stream)
+
+    def stream_fill(dst):
+        lib.cs_stream_fill(ctypes.c_void_p(dst.data_ptr()), dst.numel(), 0, stream)
+
     def wanted(name):
         return not only or name == "stream_copy" or any(name.startswith(o) for o in only)
 
@@ -195,20 +214,28 @@ def per_op_table(args, torch, ops):
         n_cold = max(2, math.ceil(600e6 / nbytes) + 1)
         n_cold = min(n_cold, 64)
         sets = [make_set() for _ in range(n_cold)]
+        op = call
+
+        def call(s_):
+            # what the op returns stays alive until this set's next turn, so the allocator hands
+            # every call a block that was last written n_cold calls ago: outputs are cold too
+            s_["_out"] = op(s_)
+
         for s in sets[:2]:
             call(s)
-        warm_med, warm_avg = event_ms(lambda i: call(sets[0]), reps, torch)
-        cold_med, cold_avg = event_ms(lambda i: call(sets[i % n_cold]), reps, torch)
+        warm_med, warm_call = event_ms(lambda i: call(sets[0]), reps, torch)
+        cold_med, cold_call = event_ms(lambda i: call(sets[i % n_cold]), reps, torch)
         rec = {
             "op": name, "config": config, "algorithmic_bytes": nbytes,
             "ms_warm": round(warm_med, 5), "ms_cold": round(cold_med, 5),
+            "ms_cold_per_call_events": round(cold_call, 5),
             "gbps_warm": round(nbytes / warm_med / 1e6, 1), "gbps_cold": round(nbytes / cold_med / 1e6, 1),
             "frac_cold": round(nbytes / cold_med / 1e6 / HBM_PEAK_GBPS, 4),
-            "buffer_sets": n_cold,
+            "buffer_sets": n_cold, "calls_per_batch": reps,
         }
         if name == "stream_copy":
             copy_points.append((nbytes, cold_med))
-        else:
+        elif not name.startswith("stream_"):
             ceiling = copy_ms_at(nbytes)
             if ceiling:
                 rec["copy_ms_same_bytes"] = round(ceiling, 5)
@@ -220,8 +247,9 @@ def per_op_table(args, torch, ops):
         del sets
         torch.cuda.empty_cache()
 
-    # ---- calibration: a plain copy moving the same number of bytes as the ops below (half read,
-    # half written).  What it reaches is the practical ceiling at that size.
+    # ---- calibration: what trivial kernels reach at the sizes of the ops below.  A plain copy
+    # moving the same number of bytes (half read, half written) is the practical ceiling of an op
+    # at that size; the read-only and write-only passes show which half limits it.
     for mb in (25, 100, 400, 1600, 3500):
         nbytes = int(mb * 1e6) // 32 * 32
 
@@ -231,6 +259,15 @@ def per_op_table(args, torch, ops):
 
         add("stream_copy", f"{mb} MB moved", nbytes, mk,
             lambda s_: stream_copy(s_["b"], s_["a"]))
+    for mb in (25, 100, 400, 3500):
+        nbytes = int(mb * 1e6) // 32 * 32
+
+        def mk1(nb=nbytes):
+            return {"a": torch.empty(nb, dtype=torch.uint8, device=dev),
+                    "o": torch.empty(max(1, lib.cs_stream_read_out_words(nb)), dtype=torch.int32, device=dev)}
+
+        add("stream_read", f"{mb} MB read", nbytes, mk1, lambda s_: stream_read(s_["a"], s_["o"]))
+        add("stream_fill", f"{mb} MB written", nbytes, mk1, lambda s_: stream_fill(s_["a"]))
 
     # ---- configuration 3: LayerNorm [8192,768] bf16, fp32 parameters
     for tag, rows, C in (("small", 8192, 768), ("xl", 16384, 1600)):
@@ -274,29 +311,32 @@ def per_op_table(args, torch, ops):
         add(f"gelu_fwd_{label}", "[8192,3072] bf16", 2 * n * 2, mk, lambda s: ops.gelu_forward(s["x"], mode))
         add(f"gelu_bwd_{label}", "[8192,3072] bf16", 3 * n * 2, mk, lambda s: ops.gelu_backward(s["dy"], s["x"], mode))
 
-    # ---- configuration 1: token + position embedding
+    # ---- configuration 1: token + position embedding.  Every buffer set has its own tables and
+    # ids: with one table for all sets the gathered rows would come from the last-level cache.
     V, T = 50257, 1024
     for tag, B, C in (("small", 8, 768), ("xl", 16, 1600)):
-        wte, wpe = randn((V, C), 0.02), randn((T, C), 0.02)
         ranks = torch.arange(1, V + 1, dtype=torch.float64, device=dev).pow(-1.1)
         for kind in ("uniform", "zipf"):
             if tag == "xl" and kind == "uniform":
                 continue
-            if kind == "uniform":
-                ids = torch.randint(0, V, (B, T), generator=g, device=dev, dtype=torch.int64)
-            else:
-                ids = torch.multinomial(ranks / ranks.sum(), B * T, replacement=True, generator=g).reshape(B, T)
             fwd_bytes = B * T * 8 + B * T * C * 2 + T * C * 2 + B * T * C * 2
             bwd_bytes = B * T * 8 + B * T * C * 2 + V * C * 2 + T * C * 2
 
-            def mk():
-                return {"dout": randn((B, T, C))}
+            def mk_ids():
+                if kind == "uniform":
+                    return torch.randint(0, V, (B, T), generator=g, device=dev, dtype=torch.int64)
+                return torch.multinomial(ranks / ranks.sum(), B * T, replacement=True, generator=g).reshape(B, T)
 
-            add("embedding_fwd", f"{tag} {kind} B{B} T{T} C{C}", fwd_bytes, mk,
-                lambda s: ops.embedding_forward_add(wte, wpe, ids))
-            add("embedding_bwd", f"{tag} {kind} B{B} T{T} C{C}", bwd_bytes, mk,
-                lambda s: ops.embedding_backward_fused(s["dout"], ids, V))
-        del wte, wpe
+            def mk_fwd():
+                return {"wte": randn((V, C), 0.02), "wpe": randn((T, C), 0.02), "ids": mk_ids()}
+
+            def mk_bwd():
+                return {"dout": randn((B, T, C)), "ids": mk_ids()}
+
+            add("embedding_fwd", f"{tag} {kind} B{B} T{T} C{C}", fwd_bytes, mk_fwd,
+                lambda s: ops.embedding_forward_add(s["wte"], s["wpe"], s["ids"]))
+            add("embedding_bwd", f"{tag} {kind} B{B} T{T} C{C}", bwd_bytes, mk_bwd,
+                lambda s: ops.embedding_backward_fused(s["dout"], s["ids"], V))
 
     # ---- configuration 0 / 4: AdamW over the GPT-2-small / XL parameter sets, one launch
     for tag, n_layer, C in (("small", 12, 768), ("xl", 48, 1600)):
@@ -314,7 +354,7 @@ def per_op_table(args, torch, ops):
         gs_ = [grad[offs[i]:offs[i + 1]] for i in range(len(sizes))]
         opt = ops.MultiTensorAdamW(ws_, gs_, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
         opt.step()
-        med, avg = event_ms(lambda i: opt.step(), reps, torch)
+        med, _ = event_ms(lambda i: opt.step(), max(5, reps // 4), torch)
         nbytes = 28 * total
         rec = {"op": "adamw_multi_tensor", "config": f"{tag} {len(sizes)} tensors {total} fp32 params",
                "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
@@ -363,7 +403,7 @@ def per_op_table(args, torch, ops):
         nbytes = 2 * N * CE_V * 2 + N * 12 + 4
         bufs = [x.clone() for _ in range(3)]
         ops.fused_classifier(bufs[0], t, CE_V, inplace=True)
-        med, avg = event_ms(lambda i: ops.fused_classifier(bufs[i % 3], t, CE_V, inplace=True), max(5, reps // 4), torch)
+        med, _ = event_ms(lambda i: ops.fused_classifier(bufs[i % 3], t, CE_V, inplace=True), max(5, reps // 4), torch)
         out.append({"op": "fused_classifier", "config": f"xl [{N},{CE_V}] bf16 stride {CE_STRIDE}",
                     "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
                     "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),

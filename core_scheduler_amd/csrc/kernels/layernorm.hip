@@ -98,19 +98,30 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
   return to_acc(r.v[i / Vec16<T>::n].e[i % Vec16<T>::n]);
 }
 
+// forward launch shape (rows a wave normalises per step, next step's rows prefetched or not)
+#ifndef CS_LN_FWD_ROWS_VPL2
+#define CS_LN_FWD_ROWS_VPL2 4
+#endif
+#ifndef CS_LN_FWD_ROWS_VPL4
+#define CS_LN_FWD_ROWS_VPL4 2
+#endif
+#ifndef CS_LN_FWD_PF
+#define CS_LN_FWD_PF true
+#endif
 constexpr int kLnThreads = 256;  // 4 waves
 // backward launch shape; the defaults are the measured best, the macros exist for tuning runs
 #ifndef CS_LN_BWD_THREADS
 #define CS_LN_BWD_THREADS 512
 #endif
+// grid caps of the backward row kernel, by 16-byte vectors per lane (the partial rows the
+// launch leaves behind are one per workgroup): 512 workgroups of 8 waves, four waves per SIMD,
+// for rows of up to 128 vectors; 256, two per SIMD, beyond (their accumulators take twice the
+// registers)
+#ifndef CS_LN_BWD_MAX_BLOCKS_VPL2
+#define CS_LN_BWD_MAX_BLOCKS_VPL2 512
+#endif
 #ifndef CS_LN_BWD_MAX_BLOCKS
 #define CS_LN_BWD_MAX_BLOCKS 256
-#endif
-#ifndef CS_LN_BWD_ROWS_VPL2
-#define CS_LN_BWD_ROWS_VPL2 2
-#endif
-#ifndef CS_LN_BWD_ROWS_VPL4
-#define CS_LN_BWD_ROWS_VPL4 1
 #endif
 constexpr int kLnBwdThreads = CS_LN_BWD_THREADS;
 
@@ -143,7 +154,7 @@ __device__ __forceinline__ void load_rows(RowSet<T, VN, VPL, R> &dst, const T *_
   }
 }
 
-template <typename TX, typename TY, typename TP, int VPL, int R>
+template <typename TX, typename TY, typename TP, int VPL, int R, bool PF>
 __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
     const TX *__restrict__ x, const TP *__restrict__ gamma, const TP *__restrict__ beta,
     TY *__restrict__ y, float *__restrict__ mean, float *__restrict__ rstd, int64_t rows, int C,
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   if (row0 >= rows) return;  // wave-uniform
 
   RowSet<TX, VN, VPL, R> cur;
-  load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
+  if constexpr (PF) load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
   float g[VPL][VN], b[VPL][VN];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
@@ -175,7 +186,11 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   const float inv_c = 1.0f / (float)C;
   for (; row0 < rows; row0 += step) {
     RowSet<TX, VN, VPL, R> nxt;
-    if (row0 + step < rows) load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
+    if constexpr (PF) {
+      if (row0 + step < rows) load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
+    } else {
+      load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
+    }
     // the R rows are independent: their reductions interleave
     float mu[R], rs[R];
 #pragma unroll
@@ -225,19 +240,27 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
         }
       }
     }
-    cur = nxt;
+    if constexpr (PF) cur = nxt;
   }
 }
 
 // ----------------------------------------------------------- fast backward
-// Same walk as the forward kernel, with dy and x prefetched one step ahead.
+// One wave per row, the row (dy and x) in registers, gamma and the per-column partial sums in
+// registers for all rows a wave visits (rows gw, gw + n_waves, ...).  No software prefetch:
+// WPE waves per SIMD are resident (the launch bound asks the compiler for that), so while one
+// wave waits for its row the others compute; measured on MI355X this beats two rows per wave
+// with the next step's rows prefetched ([8192,768] bf16: 12.3 -> 9.8 us, [16384,1600]: 32.8 ->
+// 30.3 us) because twice as many waves are in flight with half the registers each.
+// The arithmetic uses explicit fused multiply-adds (contraction is off in this file, so every
+// variant of the kernel rounds alike): 17 VALU operations per element instead of 27, which
+// matters because at 16-bit storage this kernel is as close to its VALU limit as to HBM's.
 // HAS_DRES: dx_out = dx + dresidual, the gradient add that follows LayerNorm::backward on the
 // residual stream; dx is rounded to its type first, then the sum, as two kernels would.  Only
 // instantiated for the 2-vectors-per-lane plan: wider rows have no registers left for a third
 // input, and there the add runs as its own launch.
-template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int R, bool HAS_DX,
+template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int WPE, bool HAS_DX,
           bool HAS_DP, bool HAS_DRES>
-__global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
+__global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
     const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
     float *__restrict__ partial, int64_t rows, int C, const TDX *__restrict__ dres) {
@@ -246,8 +269,7 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   constexpr int kWaves = kLnBwdThreads / kWave;
-  const int64_t gw = (int64_t)blockIdx.x * kWaves + wave;
-  const int64_t step = (int64_t)gridDim.x * kWaves * R;
+  const int64_t step = (int64_t)gridDim.x * kWaves;
   const int nvec = C / VN;
   const float inv_c = 1.0f / (float)C;
 
@@ -263,88 +285,57 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_rows_kernel(
     if (HAS_DX && lane + kWave * j < nvec) load_n<TP, VN>(gamma + (lane + kWave * j) * VN, g[j]);
   }
 
-  int64_t row0 = gw * R;
-  RowSet<TDY, VN, VPL, R> dcur;
-  RowSet<TX, VN, VPL, R> xcur;
-  float mu[R], rs[R];
-  if (row0 < rows) {
-    load_rows<TDY, VN, VPL, R>(dcur, dy, row0, rows, C, nvec, lane);
-    load_rows<TX, VN, VPL, R>(xcur, x, row0, rows, C, nvec, lane);
+  for (int64_t row = (int64_t)blockIdx.x * kWaves + wave; row < rows; row += step) {
+    RowSet<TDY, VN, VPL, 1> dcur;
+    RowSet<TX, VN, VPL, 1> xcur;
+    RowSet<TDX, VN, VPL, 1> rcur;  // this row of dresidual, in flight during the reductions
+    load_rows<TDY, VN, VPL, 1>(dcur, dy, row, rows, C, nvec, lane);
+    load_rows<TX, VN, VPL, 1>(xcur, x, row, rows, C, nvec, lane);
+    if constexpr (HAS_DRES) load_rows<TDX, VN, VPL, 1>(rcur, dres, row, rows, C, nvec, lane);
+    const float mu = mean[row], rs = rstd[row];
+    float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      mu[r] = row0 + r < rows ? mean[row0 + r] : 0.f;
-      rs[r] = row0 + r < rows ? rstd[row0 + r] : 0.f;
-    }
-  }
-  for (; row0 < rows; row0 += step) {
-    RowSet<TDY, VN, VPL, R> dnxt;
-    RowSet<TX, VN, VPL, R> xnxt;
-    RowSet<TDX, VN, VPL, R> rcur;  // this step's dresidual rows, in flight during the reductions
-    if constexpr (HAS_DRES) load_rows<TDX, VN, VPL, R>(rcur, dres, row0, rows, C, nvec, lane);
-    float nmu[R], nrs[R];
-    const int64_t nrow0 = row0 + step;
-    if (nrow0 < rows) {
-      load_rows<TDY, VN, VPL, R>(dnxt, dy, nrow0, rows, C, nvec, lane);
-      load_rows<TX, VN, VPL, R>(xnxt, x, nrow0, rows, C, nvec, lane);
+    for (int j = 0; j < VPL; ++j) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        nmu[r] = nrow0 + r < rows ? mean[nrow0 + r] : 0.f;
-        nrs[r] = nrow0 + r < rows ? rstd[nrow0 + r] : 0.f;
+      for (int k = 0; k < VN; ++k) {
+        // lanes past the row hold zeros in dy, so they add nothing
+        const float xh = (raw_get<TX, VN>(xcur.v[0][j], k) - mu) * rs;
+        const float dv = raw_get<TDY, VN>(dcur.v[0][j], k);
+        if constexpr (HAS_DP) {
+          acc_g[j][k] = __builtin_fmaf(dv, xh, acc_g[j][k]);
+          acc_b[j][k] += dv;
+        }
+        if constexpr (HAS_DX) {
+          const float gd = dv * g[j][k];
+          s1 += gd;
+          s2 = __builtin_fmaf(gd, xh, s2);
+        }
       }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (row0 + r >= rows) break;
-      float s1 = 0.f, s2 = 0.f;
+    if constexpr (HAS_DX) {
+      s1 = wave_reduce(s1, SumOp{}) * inv_c;
+      s2 = wave_reduce(s2, SumOp{}) * inv_c;
+      // x-hat and dy are unpacked again from the packed row rather than kept as floats across
+      // the reduction: half the registers, a few more VALU ops
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
+        forget_unpacked(xcur.v[0][j]);
+        forget_unpacked(dcur.v[0][j]);
+        const int idx = lane + kWave * j;
+        if (idx < nvec) {
+          float o[VN];
 #pragma unroll
-        for (int k = 0; k < VN; ++k) {
-          // lanes past the row hold zeros in dy, so they add nothing
-          const float xh = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
-          const float dv = raw_get<TDY, VN>(dcur.v[r][j], k);
-          if constexpr (HAS_DP) {
-            acc_g[j][k] += dv * xh;
-            acc_b[j][k] += dv;
+          for (int k = 0; k < VN; ++k) {
+            const float xh = (raw_get<TX, VN>(xcur.v[0][j], k) - mu) * rs;
+            const float dv = raw_get<TDY, VN>(dcur.v[0][j], k);
+            // rstd * (dy gamma - mean(dy gamma) - xhat mean(dy gamma xhat))
+            o[k] = rs * __builtin_fmaf(-xh, s2, __builtin_fmaf(dv, g[j][k], -s1));
+            if constexpr (HAS_DRES)
+              o[k] = round_through<TDX>(o[k]) + raw_get<TDX, VN>(rcur.v[0][j], k);
           }
-          if constexpr (HAS_DX) {
-            const float gd = dv * g[j][k];
-            s1 += gd;
-            s2 += gd * xh;
-          }
+          store_n<TDX, VN>(dx + row * C + (int64_t)idx * VN, o);
         }
       }
-      if constexpr (HAS_DX) {
-        s1 = wave_reduce(s1, SumOp{}) * inv_c;
-        s2 = wave_reduce(s2, SumOp{}) * inv_c;
-        // x-hat and dy are unpacked again from the packed row rather than kept as
-        // floats across the reduction: half the registers, a few more VALU ops
-#pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-          forget_unpacked(xcur.v[r][j]);
-          forget_unpacked(dcur.v[r][j]);
-          const int idx = lane + kWave * j;
-          if (idx < nvec) {
-            float o[VN];
-#pragma unroll
-            for (int k = 0; k < VN; ++k) {
-              const float xh = (raw_get<TX, VN>(xcur.v[r][j], k) - mu[r]) * rs[r];
-              const float dv = raw_get<TDY, VN>(dcur.v[r][j], k);
-              o[k] = rs[r] * (dv * g[j][k] - s1 - xh * s2);
-              if constexpr (HAS_DRES)
-                o[k] = round_through<TDX>(o[k]) + raw_get<TDX, VN>(rcur.v[r][j], k);
-            }
-            store_n<TDX, VN>(dx + (row0 + r) * C + (int64_t)idx * VN, o);
-          }
-        }
-      }
-    }
-    dcur = dnxt;
-    xcur = xnxt;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      mu[r] = nmu[r];
-      rs[r] = nrs[r];
     }
   }
 
@@ -455,13 +446,13 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_split_rows_kernel(
         const float xh = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
         const float dv = raw_get<TDY, VN>(dcur.v[j], k);
         if constexpr (HAS_DP) {
-          acc_g[j][k] += dv * xh;
+          acc_g[j][k] = __builtin_fmaf(dv, xh, acc_g[j][k]);
           acc_b[j][k] += dv;
         }
         if constexpr (HAS_DX) {
           const float gd = dv * g[j][k];
           s1 += gd;
-          s2 += gd * xh;
+          s2 = __builtin_fmaf(gd, xh, s2);
         }
       }
     }
@@ -489,7 +480,7 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_split_rows_kernel(
             for (int k = 0; k < VN; ++k) {
               const float xh = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
               const float dv = raw_get<TDY, VN>(dcur.v[j], k);
-              o[k] = rs * (dv * g[j][k] - s1 - xh * s2);
+              o[k] = rs * __builtin_fmaf(-xh, s2, __builtin_fmaf(dv, g[j][k], -s1));
             }
             store_n<TDX, VN>(dx + row * C + (int64_t)idx * VN, o);
           }
@@ -535,43 +526,43 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_split_rows_kernel(
 }
 
 // Adds `nparts` partial rows in a fixed order.  Partial rows are permuted: position
-// p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  grid (ceil(C/64), 2), block
-// (64, 16): thread (cx, ry) sums partial rows ry, ry+16, ... for one column
-// into four interleaved accumulators (so four loads are always in flight),
-// then row 0 of the block adds the 16 sub-sums in order.
+// p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  grid (ceil(C/32), 2), block
+// (32, 32): thread (cx, ry) sums partial rows ry, ry+32, ... for one column, sixteen loads in
+// flight and none of them under a condition (this launch waits for the row kernel and is all
+// latency: with 512 partial rows a thread makes one round trip), then row 0 of the block adds
+// the 32 sub-sums in order.
+constexpr int kLnFinCols = 32, kLnFinRows = 32, kLnFinInFlight = 16;
+
 template <typename TP>
-__global__ __launch_bounds__(1024) void ln_bwd_finalize_kernel(const float *__restrict__ partial,
-                                                               int nparts, TP *__restrict__ dgamma,
-                                                               TP *__restrict__ dbeta, int C,
-                                                               int vn, int accumulate) {
-  __shared__ float sub[16][64];
+__global__ __launch_bounds__(kLnFinCols *kLnFinRows) void ln_bwd_finalize_kernel(
+    const float *__restrict__ partial, int nparts, TP *__restrict__ dgamma, TP *__restrict__ dbeta,
+    int C, int vn, int accumulate) {
+  __shared__ float sub[kLnFinRows][kLnFinCols];
   const int which = blockIdx.y;
   TP *out = which == 0 ? dgamma : dbeta;
   if (out == nullptr) return;  // block-uniform
-  const int col = blockIdx.x * 64 + threadIdx.x;  // a position in the permuted row
+  const int col = blockIdx.x * kLnFinCols + threadIdx.x;  // a position in the permuted row
   float s = 0.f;
   if (col < C) {
     const float *src = partial + (int64_t)which * C + col;
     const int64_t stride = 2 * (int64_t)C;
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int p = threadIdx.y;
-    for (; p + 48 < nparts; p += 64) {
-      const float v0 = src[(int64_t)p * stride], v1 = src[(int64_t)(p + 16) * stride];
-      const float v2 = src[(int64_t)(p + 32) * stride], v3 = src[(int64_t)(p + 48) * stride];
-      a0 += v0;
-      a1 += v1;
-      a2 += v2;
-      a3 += v3;
+    for (int p0 = threadIdx.y; p0 < nparts; p0 += kLnFinRows * kLnFinInFlight) {
+      float v[kLnFinInFlight];
+#pragma unroll
+      for (int u = 0; u < kLnFinInFlight; ++u) {
+        const int p = p0 + u * kLnFinRows;
+        v[u] = src[(int64_t)(p < nparts ? p : nparts - 1) * stride];
+      }
+#pragma unroll
+      for (int u = 0; u < kLnFinInFlight; ++u) s += p0 + u * kLnFinRows < nparts ? v[u] : 0.f;
     }
-    for (; p < nparts; p += 16) a0 += src[(int64_t)p * stride];
-    s = (a0 + a1) + (a2 + a3);
   }
   sub[threadIdx.y][threadIdx.x] = s;
   __syncthreads();
   if (threadIdx.y == 0 && col < C) {
     float t = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) t += sub[r][threadIdx.x];
+    for (int r = 0; r < kLnFinRows; ++r) t += sub[r][threadIdx.x];
     const int nvec = C / vn;
     const int real = (col % nvec) * vn + col / nvec;  // the column this position stands for
     if (accumulate) t += to_acc(out[real]);
@@ -737,7 +728,6 @@ __global__ __launch_bounds__(256) void ln_bwd_param_general_kernel(
 struct FastPlan {
   int vpl = 0;       // 0: not eligible
   int fwd_rows = 1;  // rows a wave normalises per step, forward
-  int bwd_rows = 1;  // the same, backward (it holds twice the data per row)
 };
 // The widest plan whose backward kernel still has registers for a third input per row
 // (dresidual); wider rows get dx + dresidual from a second launch.
@@ -753,16 +743,13 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
   const int64_t per_lane = ceil_div(nvec, (int64_t)kWave);
   if (per_lane <= 2) {
     p.vpl = 2;
-    p.fwd_rows = 4;
-    p.bwd_rows = CS_LN_BWD_ROWS_VPL2;
+    p.fwd_rows = CS_LN_FWD_ROWS_VPL2;
   } else if (per_lane <= 4) {
     p.vpl = 4;
-    p.fwd_rows = 2;
-    p.bwd_rows = CS_LN_BWD_ROWS_VPL4;
+    p.fwd_rows = CS_LN_FWD_ROWS_VPL4;
   } else if (per_lane <= 8) {
     p.vpl = 8;
     p.fwd_rows = 1;
-    p.bwd_rows = 1;
   }
   return p;
 }
@@ -775,6 +762,7 @@ FastPlan fast_plan(int64_t C, int x_dtype) {
 #endif
 constexpr int kLnFwdMaxBlocks = CS_LN_FWD_MAX_BLOCKS;
 constexpr int kLnBwdMaxBlocks = CS_LN_BWD_MAX_BLOCKS;
+constexpr int kLnBwdMaxBlocksNarrow = CS_LN_BWD_MAX_BLOCKS_VPL2;
 
 int ln_blocks(int64_t rows, int rows_per_wave, int cap, int threads = kLnThreads) {
   const int64_t rows_per_block = (int64_t)(threads / kWave) * rows_per_wave;
@@ -790,13 +778,13 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
     if (p.vpl != 0) {
       const dim3 grid((unsigned)ln_blocks(rows, p.fwd_rows, kLnFwdMaxBlocks)), block(kLnThreads);
 #define CS_LN_FWD(VPL, R)                                                                   \
-  ln_fwd_rows_kernel<TX, TY, TP, VPL, R><<<grid, block, 0, s>>>(                            \
+  ln_fwd_rows_kernel<TX, TY, TP, VPL, R, CS_LN_FWD_PF><<<grid, block, 0, s>>>(              \
       (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean,           \
       (float *)rstd, rows, (int)C, (float)eps)
       if (p.vpl == 2) {
-        CS_LN_FWD(2, 4);
+        CS_LN_FWD(2, CS_LN_FWD_ROWS_VPL2);
       } else if (p.vpl == 4) {
-        CS_LN_FWD(4, 2);
+        CS_LN_FWD(4, CS_LN_FWD_ROWS_VPL4);
       } else {
         CS_LN_FWD(8, 1);
       }
@@ -826,7 +814,8 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   if (!fuse_dres) dres = nullptr;
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
-      const int blocks = ln_blocks(rows, p.bwd_rows, kLnBwdMaxBlocks, kLnBwdThreads);
+      const int blocks =
+          ln_blocks(rows, 1, p.vpl == 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
       // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
       const int split_blocks = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
       int blocks_used = p.vpl == 8 && want_dp ? split_blocks : blocks;  // partial rows left behind
@@ -834,27 +823,27 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
       const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
       const dim3 grid((unsigned)blocks), block(kLnBwdThreads);
-#define CS_LN_BWD(VPL, R, HAS_DX, HAS_DP, HAS_DRES)                                         \
-  ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, R, HAS_DX, HAS_DP, HAS_DRES>                    \
+#define CS_LN_BWD(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                       \
+  ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, WPE, HAS_DX, HAS_DP, HAS_DRES>                  \
       <<<grid, block, lds, s>>>((const TDY *)dy, (const TX *)x, (const float *)mean,        \
                                 (const float *)rstd, (const TP *)gamma, (TDX *)dx,          \
                                 (float *)workspace, rows, (int)C, (const TDX *)dres)
-#define CS_LN_BWD_MASK(VPL, R)                \
-  if (dx && want_dp) {                        \
-    CS_LN_BWD(VPL, R, true, true, false);     \
-  } else if (dx) {                            \
-    CS_LN_BWD(VPL, R, true, false, false);    \
-  } else {                                    \
-    CS_LN_BWD(VPL, R, false, true, false);    \
+#define CS_LN_BWD_MASK(VPL, WPE)                \
+  if (dx && want_dp) {                          \
+    CS_LN_BWD(VPL, WPE, true, true, false);     \
+  } else if (dx) {                              \
+    CS_LN_BWD(VPL, WPE, true, false, false);    \
+  } else {                                      \
+    CS_LN_BWD(VPL, WPE, false, true, false);    \
   }
       if (p.vpl == 2 && dres && want_dp) {
-        CS_LN_BWD(2, CS_LN_BWD_ROWS_VPL2, true, true, true);
+        CS_LN_BWD(2, 3, true, true, true);  // four per SIMD would spill
       } else if (p.vpl == 2 && dres) {
-        CS_LN_BWD(2, CS_LN_BWD_ROWS_VPL2, true, false, true);
+        CS_LN_BWD(2, 4, true, false, true);
       } else if (p.vpl == 2) {
-        CS_LN_BWD_MASK(2, CS_LN_BWD_ROWS_VPL2)
+        CS_LN_BWD_MASK(2, 4)
       } else if (p.vpl == 4) {
-        CS_LN_BWD_MASK(4, CS_LN_BWD_ROWS_VPL4)
+        CS_LN_BWD_MASK(4, 2)
       } else if (want_dp) {
         // 8 vectors per lane: with the dgamma/dbeta accumulators a row no longer fits one wave's
         // registers (a single-wave kernel spilled ~1 KB per lane), so two waves share each row
@@ -870,13 +859,13 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
               (TDX *)dx, (float *)workspace, rows, (int)C);
         }
       } else {
-        CS_LN_BWD(8, 1, true, false, false);
+        CS_LN_BWD(8, 2, true, false, false);
       }
 #undef CS_LN_BWD_MASK
 #undef CS_LN_BWD
       int st = launch_status();
       if (st == CS_OK && want_dp) {
-        ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)64), 2), dim3(64, 16), 0, s>>>(
+        ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)kLnFinCols), 2), dim3(kLnFinCols, kLnFinRows), 0, s>>>(
             (const float *)workspace, blocks_used, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
         st = launch_status();
       }
@@ -980,8 +969,10 @@ extern "C" int cs_add_layernorm_forward(const void *x, const void *residual, voi
 
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
-  // the fast path's largest grid: one row per pair of waves per step
-  return (size_t)ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2) * 2 * (size_t)C * sizeof(float);
+  // the fast path's largest grid: the narrow-row cap, or one row per pair of waves per step
+  const int narrow = ln_blocks(rows, 1, kLnBwdMaxBlocksNarrow, kLnBwdThreads);
+  const int split = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
+  return (size_t)(narrow > split ? narrow : split) * 2 * (size_t)C * sizeof(float);
 }
 
 namespace {
