@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // cs::compute::CrossEntropy, the reference's op interface (include/compute/cross_entropy.h:25-60).
 // forward returns the loss; backward returns the gradient of the logits (no upstream gradient
 // argument: the reference feeds ones_like(loss)).  Here forward computes both in one pass and

@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // cs::compute::LayerNorm, the reference's op interface (include/compute/layer_norm.h:24-87).
 //
 // init makes gamma = 1 and beta = 0 of `normalized_shape` (one trailing dimension here: the

@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // Task body interface (the reference's include/internal/threading/task_impl.h:23-61).
 //
 // A task is what an op call turns into: the handles it will fill (output), the handles it

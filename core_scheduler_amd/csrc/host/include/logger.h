@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // Error convention of the reference (include/logger.h:26-34): a failed
 // CS_ASSERT_TRUE logs at critical level and aborts; CS_WARN_TRUE only logs.
 // spdlog is not a dependency here: the message goes to stderr.

@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // cs::module::AdamW (the reference's include/module/adamw.h:22-41).  step() updates every
 // parameter of the module tree; where the reference submits one task and one kernel launch
 // per parameter (src/module/adamw.cpp:32-38), this one submits one task with one launch for

@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // cs::module::Embedding (the reference's include/module/embedding.h:22-39): the op's state
 // registered in a module tree ("wte.weight" in named_parameters()).  forward and backward pass
 // straight through to cs::compute::Embedding; backward returns nothing, the gradient of the

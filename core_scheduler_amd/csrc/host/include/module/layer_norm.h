@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // cs::module::LayerNorm (the reference's include/module/layer_norm.h:22-39): the op's state
 // registered in a module tree, so that its parameters appear in named_parameters() under the
 // module's path ("h.0.ln_1.weight") and an optimizer module finds them.  forward and backward

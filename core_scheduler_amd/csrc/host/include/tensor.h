@@ -1,3 +1,8 @@
+// The declarations in this header restate the public interface of CoreScheduler
+// (Copyright (c) 2024 The Core team, licensed under the Apache License, Version 2.0,
+// http://www.apache.org/licenses/LICENSE-2.0) so that code written against it compiles
+// unchanged; the comments and everything behind the declarations are this project's.
+//
 // Tensor handles of the op API (the reference's include/tensor.h:36-63).
 //
 // A handle is a shared pointer to {at::Tensor, completion event, the lane of the stream that
@@ -11,6 +16,7 @@
 #include <ATen/core/TensorBody.h>
 
 #include <memory>
+#include <ostream>
 
 #include "export.h"
 
@@ -48,6 +54,11 @@ struct Tensor : ReadOnlyTensor {
   CS_API Tensor() = default;
   CS_API void wait() const;
 };
+
+// Waits for the tensor, then prints it the way at::print does (`linesize` characters per line).
+CS_API std::ostream &print(std::ostream &stream, const ReadOnlyTensor &tensor, int64_t linesize);
+
+inline std::ostream &operator<<(std::ostream &out, const ReadOnlyTensor &t) { return print(out, t, 80); }
 }  // namespace cs
 
 // The comparisons the reference's tests use on handles: wait, then at::allclose with its defaults.

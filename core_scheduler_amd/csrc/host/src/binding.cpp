@@ -6,6 +6,7 @@
 
 #include <memory>
 #include <optional>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -72,6 +73,12 @@ PYBIND11_MODULE(_cs_host, m) {
       .def("priority", [](const ReadOnlyTensor &t) { return static_cast<int>(t.impl()->priority()); });
   py::class_<Tensor, ReadOnlyTensor>(m, "Tensor").def(py::init<>());
 
+  // operator<< of a handle (include/tensor.h): waits, then at::print with 80 characters per line
+  m.def("tensor_to_string", [](const ReadOnlyTensor &t) {
+    std::ostringstream out;
+    out << t;
+    return out.str();
+  }, py::arg("tensor"));
   m.def("to_torch", &memory::to_torch, py::arg("scheduler"), py::arg("tensor"));
   m.def("clip_grad_norm_", &compute::Utils::clip_grad_norm_, py::arg("scheduler"), py::arg("tensors"),
         py::arg("max_norm"), py::arg("norm_type") = 2.0);

@@ -157,7 +157,8 @@ void AdamWImpl::step(const Scheduler &scheduler) const {
     CS_ASSERT_TRUE(state != nullptr, "not an AdamW state: " + kv.key());
     const auto *increment = increments.find(kv.key());
     CS_ASSERT_TRUE(increment != nullptr, "parameter " + kv.key() + " is no longer in the module");
-    increment->parameter.wait();  // its dtype is read below
+    // no host wait: the handle's at::Tensor exists since the task that made it was submitted
+    // (tasks run inline on the submitting thread), and only its dtype is read here
     const auto &o = state->options;
     const Key key{static_cast<int>(increment->parameter.impl()->tensor().scalar_type()), o.lr, o.beta1, o.beta2,
                   o.eps, o.weight_decay, o.amsgrad, o.t};

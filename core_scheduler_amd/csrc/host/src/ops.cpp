@@ -6,6 +6,7 @@
 #include <ATen/autocast_mode.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <ATen/ops/empty.h>
+#include <ATen/ops/add.h>
 #include <ATen/ops/empty_like.h>
 #include <ATen/ops/normal.h>
 #include <ATen/ops/ones.h>
@@ -223,14 +224,14 @@ std::shared_ptr<Embedding::State> Embedding::init(const Scheduler &scheduler, co
   int64_t padding_idx = -1;
   if (options.padding_idx().has_value()) {
     const int64_t p = *options.padding_idx();
+    // As in the reference (src/compute/embedding.cpp:80-90): a positive index is only checked
+    // and a zero one ignored, so State::Args::padding_idx stays -1 for both and that row keeps
+    // its gradient; only a negative index is normalised and takes effect in backward.
     if (p > 0) {
       TORCH_CHECK(p < options.num_embeddings(), "Padding_idx must be within num_embeddings");
-      padding_idx = p;
     } else if (p < 0) {
       TORCH_CHECK(p >= -options.num_embeddings(), "Padding_idx must be within num_embedding");
       padding_idx = options.num_embeddings() + p;
-    } else {
-      padding_idx = 0;
     }
   }
   TORCH_CHECK(!options.max_norm().has_value(), "max_norm is not supported");
@@ -282,6 +283,11 @@ void Embedding::backward(const Scheduler &scheduler, const std::shared_ptr<State
       const bool accumulate = gw.defined();  // `=` for a fresh gradient, `+=` otherwise
       const int64_t C = dout.size(-1);
       if (!accumulate) gw = at::empty({args.num_weights, C}, dout.options());
+      // the kernel adds into the existing gradient with dout's element type and row length
+      TORCH_CHECK(gw.scalar_type() == dout.scalar_type() && gw.dim() == 2 && gw.size(0) == args.num_weights &&
+                      gw.size(1) == C && gw.is_contiguous(),
+                  "Embedding::backward: the existing gradient must be a contiguous [num_embeddings, C] tensor of "
+                  "grad_output's dtype");
       at::Tensor ws = workspace(cs_embedding_backward_workspace_bytes(idx.numel(), C, args.num_weights), dout);
       check(cs_embedding_backward(dout.data_ptr(), idx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws.numel(),
                                   idx.numel(), C, args.num_weights, args.padding_idx, dtype_of(dout.scalar_type()),
@@ -467,25 +473,45 @@ Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<Sta
       at::Tensor dy = T(input()[0]).contiguous();
       const at::Tensor mean = T(input()[2]), rstd = T(input()[3]);
       const at::Tensor g = T(input()[4]).contiguous();
-      // dy is either x's type or fp32 (autocast); anything else is brought to x's type
-      if (dy.scalar_type() != x.scalar_type() && dy.scalar_type() != at::kFloat) dy = dy.to(x.scalar_type());
+      // dy is either x's type or fp32 (autocast over 16-bit x); anything else is brought to x's type
+      const bool narrow_x = x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16;
+      if (dy.scalar_type() != x.scalar_type() && !(narrow_x && dy.scalar_type() == at::kFloat))
+        dy = dy.to(x.scalar_type());
       const int64_t C = x.size(-1), rows = x.numel() / C;
       at::Tensor dx = at::empty(x.sizes(), x.options().dtype(dy.scalar_type()));
       at::Tensor &gw = T(output()[1]);
       at::Tensor *gb = has_bias ? &T(output()[2]) : nullptr;
       const bool accumulate = gw.defined();  // += into gradients that already exist
       if (has_bias) CS_ASSERT_TRUE(gb->defined() == accumulate, "weight and bias gradients must exist together");
-      if (!accumulate) {
-        gw = at::empty({C}, g.options());
-        if (has_bias) *gb = at::empty({C}, g.options());
+      // fp32 dy with 16-bit parameters (autocast over a model whose LayerNorm weights are 16 bit):
+      // the kernels take fp32 parameters with fp32 dy, so gamma is widened and the parameter
+      // gradients come out in fp32 and are narrowed (or added) afterwards, [C] elements each
+      const bool widen = dy.scalar_type() == at::kFloat && g.scalar_type() != at::kFloat && narrow_x;
+      const at::Tensor gk = widen ? g.to(at::kFloat) : g;
+      at::Tensor dgk, dbk;
+      if (widen || !accumulate) {
+        // an empty batch leaves the gradients untouched: they are zero then
+        dgk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
+        if (has_bias) dbk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
+      } else {
+        dgk = gw;
+        if (has_bias) dbk = *gb;
       }
+      const bool kernel_accumulates = accumulate && !widen;
       at::Tensor ws = workspace(cs_layernorm_backward_workspace_bytes(rows, C), x);
-      check(cs_layernorm_backward(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), g.data_ptr(),
-                                  dx.data_ptr(), gw.data_ptr(), has_bias ? gb->data_ptr() : nullptr, ws.data_ptr(),
+      check(cs_layernorm_backward(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), gk.data_ptr(),
+                                  dx.data_ptr(), dgk.data_ptr(), has_bias ? dbk.data_ptr() : nullptr, ws.data_ptr(),
                                   ws.numel(), rows, C, dtype_of(dy.scalar_type()), dtype_of(x.scalar_type()),
-                                  dtype_of(dx.scalar_type()), dtype_of(g.scalar_type()), accumulate ? 1 : 0,
+                                  dtype_of(dx.scalar_type()), dtype_of(gk.scalar_type()), kernel_accumulates ? 1 : 0,
                                   current_stream()),
             name());
+      if (widen) {
+        gw = accumulate ? gw + dgk.to(g.scalar_type()) : dgk.to(g.scalar_type());
+        if (has_bias) *gb = accumulate ? *gb + dbk.to(g.scalar_type()) : dbk.to(g.scalar_type());
+      } else if (!accumulate) {
+        gw = dgk;
+        if (has_bias) *gb = dbk;
+      }
       T(output()[0]) = dx;
     }
     [[nodiscard]] const char *name() const override { return "cs::compute::LayerNorm::backward"; }
@@ -574,6 +600,18 @@ Tensor clip_grad_norm_(const Scheduler &scheduler, const std::vector<Tensor> &te
 
 // =================================================================== AdamW
 namespace optimizer {
+namespace {
+// The kernels take one element type and one count for the parameter, its gradient and its state
+// (the reference's data_ptr<T>() throws on a mismatch, src/optimizer/adamw.cu:96-103).
+void check_adamw_tensors(const at::Tensor &g, const at::Tensor &w, const at::Tensor &m, const at::Tensor &v,
+                         const at::Tensor *v_max) {
+  const auto same = [&](const at::Tensor &t) { return t.scalar_type() == g.scalar_type() && t.numel() == g.numel(); };
+  TORCH_CHECK(same(w) && same(m) && same(v) && (v_max == nullptr || same(*v_max)),
+              "AdamW: the parameter, its gradient and its state must share one dtype and element count (gradient ",
+              g.scalar_type(), " x ", g.numel(), ", parameter ", w.scalar_type(), " x ", w.numel(), ")");
+}
+}  // namespace
+
 AdamW::State::State(const Tensors &tensors, const Options &options) : tensors{tensors}, options{options} {}
 void AdamW::State::set_lr(const double lr) const { options.lr = lr; }
 double AdamW::State::get_lr() const { return options.lr; }
@@ -613,6 +651,7 @@ void AdamW::step(const Scheduler &scheduler, const std::shared_ptr<module::Optim
       }
       at::Tensor &w = T(output()[0]), &m = T(output()[1]), &v = T(output()[2]);
       TORCH_CHECK(w.is_contiguous() && m.is_contiguous() && v.is_contiguous(), "AdamW needs contiguous state");
+      check_adamw_tensors(g, w, m, v, options.amsgrad ? &T(output()[3]) : nullptr);
       const at::Tensor gc = g.contiguous();
       check(cs_adamw_step(w.data_ptr(), gc.data_ptr(), m.data_ptr(), v.data_ptr(),
                           options.amsgrad ? T(output()[3]).data_ptr() : nullptr, gc.numel(),
@@ -668,6 +707,7 @@ Tensor AdamW::step(const Scheduler &scheduler, const std::vector<std::shared_ptr
         at::Tensor &w = T(output()[4 * i]), &m = T(output()[4 * i + 1]), &v = T(output()[4 * i + 2]);
         TORCH_CHECK(g.is_contiguous() && w.is_contiguous() && m.is_contiguous() && v.is_contiguous(),
                     "multi-tensor AdamW needs contiguous tensors");
+        check_adamw_tensors(g, w, m, v, options.amsgrad ? &T(output()[4 * i + 3]) : nullptr);
         const int dt = dtype_of(g.scalar_type());
         CS_ASSERT_TRUE(dtype < 0 || dt == dtype, "multi-tensor AdamW needs one dtype");
         dtype = dt;

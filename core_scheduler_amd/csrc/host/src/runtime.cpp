@@ -24,6 +24,7 @@
 #include "threading/event.h"
 #include "threading/scheduler_impl.h"
 #include "threading/task_impl.h"
+#include "trace_range.h"
 
 namespace cs {
 // ------------------------------------------------------------------ events
@@ -88,6 +89,10 @@ void ReadOnlyTensor::wait() const { impl_->event().synchronize(); }
 const std::shared_ptr<ReadOnlyTensor::Impl> &ReadOnlyTensor::impl() const { return impl_; }
 void ReadOnlyTensor::reset() { impl_ = std::make_shared<Impl>(); }
 void Tensor::wait() const { ReadOnlyTensor::wait(); }
+std::ostream &print(std::ostream &stream, const ReadOnlyTensor &tensor, const int64_t linesize) {
+  tensor.wait();
+  return at::print(stream, tensor.impl()->tensor(), linesize);
+}
 
 // ------------------------------------------------------------------- tasks
 Task::Task(std::shared_ptr<Impl> impl) : impl_{std::move(impl)} {}
@@ -155,7 +160,11 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
     for (const auto &t : task.impl()->input()) {
       if (t.impl()->priority() != lane && !t.impl()->event().query()) t.impl()->event().block();
     }
-    task();
+    {
+      // the task's name as a range in marker traces (rocprofv3 --marker-trace)
+      const TraceRange range{task.impl()->name()};
+      task();
+    }
     for (const auto &t : task.impl()->output()) {
       t.impl()->priority() = lane;
       t.impl()->event().record();

@@ -11,7 +11,7 @@
 // does ~20 flops, so it is bound by HBM: every lane moves 16 B per access
 // (non-temporal: +6% over plain loads here),
 // each workgroup owns one contiguous chunk, and nothing is read twice.
-#include "common.cuh"
+#include "common.hpp"
 
 #include <math.h>
 

@@ -1,6 +1,6 @@
 // Version and error reporting of the C ABI, and the plain copy kernel used to
 // calibrate bandwidth measurements.
-#include "common.cuh"
+#include "common.hpp"
 
 namespace cs_hip {
 namespace {

@@ -22,7 +22,7 @@
 //   fp64, unaligned base pointers    ce_rows_general_kernel
 // Probabilities are 2^(x*log2e - max*log2e) / sum with one fma and one hardware exp2 per
 // element; the row loss is ln(sum) - (x_t - max).
-#include "common.cuh"
+#include "common.hpp"
 
 #include <math.h>
 

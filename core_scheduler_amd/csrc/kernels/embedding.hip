@@ -33,7 +33,7 @@
 // fill and the position-table sum next to that.
 // The traffic that matters is the dense write of dweight (V*C elements), one
 // read of dout and a second write of the indexed rows.
-#include "common.cuh"
+#include "common.hpp"
 
 #include <atomic>
 #include <type_traits>

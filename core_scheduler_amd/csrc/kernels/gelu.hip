@@ -12,7 +12,7 @@
 // exp2 and reciprocal (1 ulp each, far inside the 8-bit mantissa of the
 // result); the exact form uses an erfc polynomial for 16-bit storage (see below);
 // fp32/fp64 storage uses libm and ATen's expression as written.
-#include "common.cuh"
+#include "common.hpp"
 
 #include <math.h>
 

@@ -22,7 +22,7 @@
 // Anything the fast path cannot take (C not a multiple of the vector width,
 // C beyond the register budget, unaligned pointers, fp64) goes through a
 // plain one-workgroup-per-row path.
-#include "common.cuh"
+#include "common.hpp"
 
 #include <math.h>
 

@@ -58,8 +58,23 @@ def _workspace(nbytes, dev):
 
 
 # ------------------------------------------------------------------ AdamW
+def _check_adamw_tensors(w, dw, m, v, v_max=None):
+    """The kernels take one element type and one count for the parameter, its gradient and its
+    state; a mismatch would read or write past the end of the smaller tensor."""
+    for name, t in (("gradient", dw), ("m", m), ("v", v), ("v_max", v_max)):
+        if t is None:
+            continue
+        if t.dtype != w.dtype or t.numel() != w.numel():
+            raise ValueError(f"AdamW: {name} is {t.dtype} x {t.numel()}, the parameter {w.dtype} x {w.numel()}")
+        if not t.is_contiguous():
+            raise ValueError(f"AdamW: {name} must be contiguous")
+    if not w.is_contiguous():
+        raise ValueError("AdamW: the parameter must be contiguous")
+
+
 def adamw_step(w, dw, m, v, *, lr, beta1, beta2, eps, weight_decay, t, v_max=None):
     """One AdamW step on one tensor, in place (cs::optimizer::AdamW::step).  `t` >= 1."""
+    _check_adamw_tensors(w, dw, m, v, v_max)
     dev = _dev(w, dw, m, v, v_max)
     lib = _capi.load()
     with torch.cuda.device(dev):
@@ -81,39 +96,49 @@ class MultiTensorAdamW:
         self.params = list(params)
         self.lr, self.beta1, self.beta2, self.eps, self.weight_decay = lr, beta1, beta2, eps, weight_decay
         self.amsgrad, self.t = amsgrad, t
-        self.dev = _dev(*self.params)
         self.dtype = self.params[0].dtype
+        for p in self.params:
+            if p.dtype != self.dtype or not p.is_contiguous():
+                raise ValueError("MultiTensorAdamW needs contiguous parameters of one dtype")
+        self.dev = _dev(*self.params)
         self.m = [torch.zeros_like(p) for p in self.params]
         self.v = [torch.zeros_like(p) for p in self.params]
         self.v_max = [torch.zeros_like(p) for p in self.params] if amsgrad else None
         lib = _capi.load()
         self._bytes = lib.cs_adamw_multi_table_bytes(len(self.params))
-        self._host = torch.empty(self._bytes, dtype=torch.uint8, pin_memory=True)
         self._table = torch.empty(self._bytes, dtype=torch.uint8, device=self.dev)
         self._slots = 0
         self.refresh(grads)
 
     def refresh(self, grads):
         grads = list(grads)
+        n = len(self.params)
+        if len(grads) != n:
+            raise ValueError("one gradient per parameter")
+        for p, g in zip(self.params, grads):
+            if g.numel() != p.numel() or g.dtype != p.dtype or not g.is_contiguous():
+                raise ValueError("gradient does not match its parameter")
         _dev(*grads)
         lib = _capi.load()
-        n = len(self.params)
         arr = (_capi.AdamWTensor * n)()
         for i, (p, g) in enumerate(zip(self.params, grads)):
-            if g.numel() != p.numel() or g.dtype != p.dtype:
-                raise ValueError("gradient does not match its parameter")
             arr[i].w, arr[i].dw = p.data_ptr(), g.data_ptr()
             arr[i].m, arr[i].v = self.m[i].data_ptr(), self.v[i].data_ptr()
             arr[i].v_max = self.v_max[i].data_ptr() if self.amsgrad else None
             arr[i].n = p.numel()
         slots = ctypes.c_int64(0)
-        code = lib.cs_adamw_multi_build_table(arr, n, _DTYPES[self.dtype],
-                                              ctypes.c_void_p(self._host.data_ptr()), self._bytes,
-                                              ctypes.byref(slots))
+        # A new pinned block for every refresh: the copy below reads it when the stream gets
+        # there, not now, and the host may be a step ahead of the device; rewriting one shared
+        # block would hand the step still queued the next step's gradient addresses.  The block
+        # goes back to torch's pinned allocator, which reuses it only after the copy has run.
+        host = torch.empty(self._bytes, dtype=torch.uint8, pin_memory=True)
+        code = lib.cs_adamw_multi_build_table(arr, n, _DTYPES[self.dtype], ctypes.c_void_p(host.data_ptr()),
+                                              self._bytes, ctypes.byref(slots))
         _capi.check("cs_adamw_multi_build_table", code)
         self._slots = slots.value
         self._grads = grads  # keep them alive: the table holds their addresses
-        self._table.copy_(self._host, non_blocking=True)
+        with torch.cuda.device(self.dev):
+            self._table.copy_(host, non_blocking=True)
 
     def step(self, max_grad_norm=None, norm_type=2.0):
         """One launch for every parameter.  With `max_grad_norm`, the global gradient norm is
@@ -294,12 +319,20 @@ def embedding_forward_add(wte, wpe, indices):
     return out
 
 
+def _check_table_gradient(t, rows, C, dtype, name):
+    """An existing gradient is added to with dout's element type and row length."""
+    if t.dtype != dtype or tuple(t.shape) != (rows, C) or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous [{rows}, {C}] tensor of {dtype}, got {tuple(t.shape)} {t.dtype}")
+
+
 def embedding_backward(dout, indices, num_weights, padding_idx=-1, dweight=None):
     """Dense dweight [num_weights, C]; passing dweight accumulates into it."""
-    dev = _dev(dout, indices, dweight)
     C = dout.shape[-1]
     n = indices.numel()
     accumulate = dweight is not None
+    if accumulate:
+        _check_table_gradient(dweight, num_weights, C, dout.dtype, "dweight")
+    dev = _dev(dout, indices, dweight)
     if dweight is None:
         dweight = torch.empty(num_weights, C, dtype=dout.dtype, device=dev)
     lib = _capi.load()
@@ -315,11 +348,14 @@ def embedding_backward(dout, indices, num_weights, padding_idx=-1, dweight=None)
 
 def embedding_backward_fused(dout, indices, num_weights, dwte=None, dwpe=None):
     """(dwte, dwpe) of out = wte[ids] + wpe[pos] from dout [B,T,C]."""
-    dev = _dev(dout, indices, dwte, dwpe)
     B, T, C = dout.shape
     accumulate = dwte is not None
     if (dwte is None) != (dwpe is None):
         raise ValueError("pass both gradients to accumulate, or neither")
+    if accumulate:
+        _check_table_gradient(dwte, num_weights, C, dout.dtype, "dwte")
+        _check_table_gradient(dwpe, T, C, dout.dtype, "dwpe")
+    dev = _dev(dout, indices, dwte, dwpe)
     if dwte is None:
         dwte = torch.empty(num_weights, C, dtype=dout.dtype, device=dev)
         dwpe = torch.empty(T, C, dtype=dout.dtype, device=dev)
@@ -335,9 +371,11 @@ def embedding_backward_fused(dout, indices, num_weights, dwte=None, dwpe=None):
 
 
 def embedding_backward_positions(dout, dwpe=None):
-    dev = _dev(dout, dwpe)
     B, T, C = dout.shape
     accumulate = dwpe is not None
+    if accumulate:
+        _check_table_gradient(dwpe, T, C, dout.dtype, "dwpe")
+    dev = _dev(dout, dwpe)
     if dwpe is None:
         dwpe = torch.empty(T, C, dtype=dout.dtype, device=dev)
     with torch.cuda.device(dev):

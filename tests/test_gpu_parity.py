@@ -126,6 +126,29 @@ def test_adamw_multi_tensor_small_set(ops, co):
         assert_bit_exact(gws[i], flat[i], f"multi == flat [{i}]")  # same arithmetic, two launch shapes
 
 
+def test_adamw_multi_tensor_refresh_back_to_back_uses_each_steps_own_gradients(ops):
+    """Gradients are re-allocated every step, so the descriptor table is rebuilt and uploaded
+    every step while the host runs ahead of the device: each queued step must see the table
+    that was built for it, not a later one."""
+    n = 1 << 20
+    w = dev(randn(n, 70, std=0.02))
+    ref = w.clone()
+    grads = [dev(randn(n, 71 + i, std=1e-3)) for i in range(6)]
+    opt = ops.MultiTensorAdamW([w], [grads[0]], t=0, **HYPER)
+    m, v = torch.zeros_like(ref), torch.zeros_like(ref)
+    blocker_a = torch.empty(1 << 28, dtype=torch.uint8, device=DEV)
+    blocker_b = torch.empty_like(blocker_a)
+    for _ in range(8):
+        blocker_b.copy_(blocker_a)  # the device is busy while the host queues all six steps
+    for g in grads:
+        opt.refresh([g])
+        opt.step()
+    torch.cuda.synchronize()
+    for t, g in enumerate(grads, 1):
+        ops.adamw_step(ref, g, m, v, t=t, **HYPER)
+    assert_bit_exact(w, ref, "six queued steps, one table upload each")
+
+
 def test_adamw_gpt2_small_ten_steps(ops, co):
     """Benchmark configuration 0: all 148 GPT-2-small tensors, 10 steps, fresh grads each step."""
     shapes = gpt2_param_shapes()

@@ -247,6 +247,49 @@ def test_layer_norm_autocast_and_no_bias(host, sched, co):
     assert nb.grad_weight.defined() and not nb.grad_bias.defined()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
+def test_layer_norm_autocast_with_16_bit_parameters(host, sched, co, dtype):
+    # a model whose LayerNorm parameters are 16 bit, run inside the autocast guard: fp32 y, fp32 dy and dx,
+    # parameter gradients in the parameters' type, twice (the second backward adds to the first)
+    td = getattr(torch, dtype)
+    x = randn((4, 32, 768), 21, dtype=td)
+    dy = randn((4, 32, 768), 22)
+    state = host.LayerNorm.init(sched, [768], dtype=dtype)
+    gamma, beta = randn(768, 23, std=0.02, mean=1.0, dtype=td), randn(768, 24, std=0.02, dtype=td)
+    state.set_weight(up(host, sched, gamma))
+    state.set_bias(up(host, sched, beta))
+    scope = host.autocast()
+    scope.enter(sched, dtype)
+    try:
+        y = host.LayerNorm.forward(sched, state, up(host, sched, x))
+        dx = host.LayerNorm.backward(sched, state, up(host, sched, dy))
+        host.LayerNorm.forward(sched, state, up(host, sched, x))
+        host.LayerNorm.backward(sched, state, up(host, sched, dy))
+    finally:
+        scope.exit()
+    x2, g2, b2 = x.reshape(-1, 768), gamma.float(), beta.float()
+    y2, mean, rstd = co.layernorm_forward(x2, g2, b2, out_dtype=torch.float32)
+    dx2, dg2, db2 = co.layernorm_backward(dy.reshape(-1, 768), x2, mean, rstd, g2, out_dtype=torch.float32)
+    assert_close(down(host, sched, y).reshape(-1, 768), y2, atol=2e-6, name="y fp32")
+    assert_close(down(host, sched, dx).reshape(-1, 768), dx2, atol=5e-6, name="dx fp32")
+    got_dg, got_db = down(host, sched, state.grad_weight), down(host, sched, state.grad_bias)
+    assert got_dg.dtype == td and got_db.dtype == td
+    # each backward's gradient is rounded to 16 bit, then the two are added and rounded again
+    want_dg = (dg2.to(td).float() * 2).to(td)
+    want_db = (db2.to(td).float() * 2).to(td)
+    assert_close(got_dg, want_dg, atol=1e-4, name="dgamma, two backward passes")
+    assert_close(got_db, want_db, atol=1e-4, name="dbeta, two backward passes")
+
+
+@pytest.mark.gpu
+def test_tensor_handles_print_like_at_print(host, sched):
+    # include/tensor.h:65-70: print waits for the tensor and hands it to at::print
+    t = up(host, sched, torch.tensor([[1.0, 2.5, -3.0], [4.0, 0.0, 6.0]]))
+    text = host.tensor_to_string(t)
+    assert "2.5" in text and "-3" in text and "{2,3}" in text, text
+
+
 # -------------------------------------------------------------------------- AdamW
 @pytest.mark.gpu
 @pytest.mark.parametrize("size", [128, 512, 1024])
@@ -505,6 +548,46 @@ def test_embedding_argument_checks_raise():
                 print("raised:", str(e).splitlines()[0])
     """)
     assert p.stdout.count("raised:") == 3, p.stdout + p.stderr
+
+
+def test_layer_norm_without_affine_parameters_aborts_like_the_reference():
+    # src/compute/layer_norm.cpp:78-79: CS_ASSERT_TRUE(elementwise_affine) -> log critical + std::abort
+    p = run_snippet("""
+        from core_scheduler_amd import _cs_host as h
+        h.LayerNorm.init(h.Scheduler(), [8], elementwise_affine=False)
+    """)
+    assert p.returncode != 0 and "elementwise_affine" in (p.stderr + p.stdout)
+
+
+@pytest.mark.gpu
+def test_padding_idx_state_matches_the_reference(host, sched):
+    # src/compute/embedding.cpp:80-90
+    assert host.Embedding.init(sched, 10, 4, padding_idx=3).padding_idx == -1
+    assert host.Embedding.init(sched, 10, 4, padding_idx=0).padding_idx == -1
+    assert host.Embedding.init(sched, 10, 4, padding_idx=-2).padding_idx == 8
+    assert host.Embedding.init(sched, 10, 4).padding_idx == -1
+
+
+@pytest.mark.gpu
+def test_exception_in_a_main_stream_task_aborts_and_names_the_task():
+    # src/threading/dynamic_scheduler.cpp:176-195: a std::exception escaping a kMain task body becomes
+    # log critical + std::abort with the task's name.  Float indices make Embedding::forward's body throw
+    # (TORCH_CHECK) before it launches anything; the device is idle when the process aborts.
+    p = run_snippet("""
+        import torch
+        from core_scheduler_amd import _cs_host as h
+        s = h.DynamicScheduler(0)
+        state = h.Embedding.init(s, 10, 4)
+        state.weight.wait()
+        idx = h.from_torch(s, torch.zeros(2, 3, device="cuda:0"))
+        idx.wait()
+        torch.cuda.synchronize()
+        h.Embedding.forward(s, state, idx)
+        print("not reached")
+    """)
+    out = p.stdout + p.stderr
+    assert p.returncode != 0 and "not reached" not in out, out
+    assert "cs::compute::Embedding::forward" in out and "int32 or int64" in out, out
 
 
 def test_module_names_are_checked():
