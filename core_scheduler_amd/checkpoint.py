@@ -10,8 +10,9 @@ looks each key up in `named_parameters()` (an unknown key is an error), and copi
 The reference leaves optimizer checkpoints unimplemented
 (src/module/optimizer_module.cpp:45-51); `save_optimizer` / `load_optimizer` write AdamW's
 first and second moments (and v_max) in the same layout under "<parameter>.m", ".v", ".v_max",
-plus one row "<parameter>.t" holding the step count, so that a run can resume with the state
-it stopped with.
+plus one row "<parameter>.t" holding the step count as two floats (t mod 2^24, t div 2^24, both
+exact in float32), so that a run can resume with the state it stopped with.  The C++ host
+library writes and reads the same files (cs::save / cs::load in csrc/host/src/checkpoint.cpp).
 
 Everything here is host-side file work on torch tensors; nothing touches a kernel.
 """
@@ -20,6 +21,8 @@ from collections import OrderedDict
 import pyarrow as pa
 import pyarrow.parquet as pq
 import torch
+
+T_SPLIT = 1 << 24  # float32 holds every integer up to here
 
 SCHEMA = pa.schema([pa.field("key", pa.utf8()), pa.field("value", pa.list_(pa.field("item", pa.float32())))])
 
@@ -84,7 +87,8 @@ def save_optimizer(named_states, path):
         rows.append((f"{name}.v", state["v"]))
         if state.get("v_max") is not None:
             rows.append((f"{name}.v_max", state["v_max"]))
-        rows.append((f"{name}.t", torch.tensor([float(state["t"])])))
+        t = int(state["t"])
+        rows.append((f"{name}.t", torch.tensor([float(t % T_SPLIT), float(t // T_SPLIT)])))
     save_tensors(rows, path)
 
 
@@ -96,5 +100,8 @@ def load_optimizer(path):
         if field not in ("m", "v", "v_max", "t"):
             raise KeyError(f"not an optimizer checkpoint row: {key}")
         entry = out.setdefault(name, {"m": None, "v": None, "v_max": None, "t": 0})
-        entry[field] = int(flat.item()) if field == "t" else flat
+        if field == "t":  # one value in files written before the count was split
+            entry[field] = int(round(flat[0].item())) + (int(round(flat[1].item())) * T_SPLIT if flat.numel() > 1 else 0)
+        else:
+            entry[field] = flat
     return out

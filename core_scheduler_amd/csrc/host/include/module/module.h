@@ -75,3 +75,26 @@ std::shared_ptr<ModuleType> Module::register_module(std::string name,
   return register_module(std::move(name), module_holder.ptr());
 }
 }  // namespace cs::module
+
+// Checkpoints in the reference's Parquet layout (the reference's include/module/module.h:92-108,
+// src/module/module.cpp:129-220): one row per parameter, `key` = qualified name, `value` = the
+// parameter flattened as float32.  load copies every row of the file into the parameter of that
+// name (converted to its dtype, device and shape); a name the module does not have aborts.
+// Both wait for the tensors they touch; the second form takes a holder (cs::module::LayerNorm).
+namespace cs {
+CS_API void save(const module::Module &module, const std::string &path);
+
+template <typename Module, typename = std::enable_if_t<!std::is_base_of_v<module::Module, Module> &&
+                                                       !std::is_base_of_v<ReadOnlyTensor, Module>>>
+static void save(const Module &module, const std::string &path) {
+  save(*module, path);
+}
+
+CS_API void load(const module::Module &module, const std::string &path);
+
+template <typename Module, typename = std::enable_if_t<!std::is_base_of_v<module::Module, Module> &&
+                                                       !std::is_base_of_v<ReadOnlyTensor, Module>>>
+static void load(const Module &module, const std::string &path) {
+  load(*module, path);
+}
+}  // namespace cs

@@ -29,3 +29,11 @@ struct CS_API OptimizerModule : std::enable_shared_from_this<OptimizerModule> {
   std::weak_ptr<const Module> module_;
 };
 }  // namespace cs::module
+
+// Optimizer checkpoints (declared in the reference's include/module/optimizer_module.h:54-60; its
+// definitions abort with "not implemented", src/module/optimizer_module.cpp:45-51).  Here:
+// AdamW's m, v (and v_max) and step count per parameter, in the layout of cs::save(Module).
+namespace cs {
+CS_API void save(const module::OptimizerModule &module, const std::string &path);
+CS_API void load(const module::OptimizerModule &module, const std::string &path);
+}  // namespace cs

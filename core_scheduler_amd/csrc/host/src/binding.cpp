@@ -207,6 +207,15 @@ PYBIND11_MODULE(_cs_host, m) {
       Op::step(s, base, ws, grads);
     });
   }
+  // ---- checkpoints (cs::save / cs::load, include/module/module.h and optimizer_module.h)
+  m.def("save_module", [](const std::shared_ptr<module::Module> &mod, const std::string &path) { cs::save(*mod, path); },
+        py::arg("module"), py::arg("path"));
+  m.def("load_module", [](const std::shared_ptr<module::Module> &mod, const std::string &path) { cs::load(*mod, path); },
+        py::arg("module"), py::arg("path"));
+  m.def("save_optimizer", [](const std::shared_ptr<module::AdamWImpl> &opt, const std::string &path) { cs::save(static_cast<const module::OptimizerModule &>(*opt), path); },
+        py::arg("optimizer"), py::arg("path"));
+  m.def("load_optimizer", [](const std::shared_ptr<module::AdamWImpl> &opt, const std::string &path) { cs::load(static_cast<const module::OptimizerModule &>(*opt), path); },
+        py::arg("optimizer"), py::arg("path"));
   // ---- module layer
   {
     using module::Module;

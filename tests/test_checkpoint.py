@@ -55,6 +55,13 @@ def test_unknown_key_is_an_error_and_missing_ones_are_left_alone(tmp_path):
         ck.load_into({"a": torch.zeros(4)}, path)
 
 
+def test_step_counts_beyond_float_precision_survive(tmp_path):
+    path = str(tmp_path / "opt.parquet")
+    t = (1 << 24) * 5 + 12345  # not representable in one float32
+    ck.save_optimizer([("w", {"m": torch.zeros(2), "v": torch.zeros(2), "v_max": None, "t": t})], path)
+    assert ck.load_optimizer(path)["w"]["t"] == t
+
+
 def test_optimizer_state_round_trip(tmp_path):
     path = str(tmp_path / "opt.parquet")
     states = [("wte.weight", {"m": torch.randn(5, 4), "v": torch.rand(5, 4), "v_max": None, "t": 17}),
@@ -88,3 +95,82 @@ def test_module_tree_round_trip_on_the_gpu(tmp_path):
     for k, p in root.named_parameters():
         assert torch.equal(host.to_torch(sched, p).cpu(), before[k]), k
     assert os.path.getsize(path) > 0
+
+
+def _tree(host, sched):
+    root = host.Container()
+    root.register_module("wte", host.EmbeddingModule(sched, 50, 16))
+    h = root.register_module("h", host.Container())
+    h.register_module("ln_1", host.LayerNormModule(sched, [16]))
+    return root
+
+
+@pytest.mark.gpu
+def test_cpp_save_is_read_by_python_and_python_files_by_cpp_load(tmp_path):
+    """cs::save / cs::load (the C++ host library, Arrow C++) against checkpoint.py (pyarrow): either
+    side reads what the other wrote, values bit-equal, same schema, one row group."""
+    from core_scheduler_amd import _cs_host as host
+
+    sched = host.DynamicScheduler(0)
+    root = _tree(host, sched)
+    before = {k: host.to_torch(sched, p).cpu() for k, p in root.named_parameters()}
+    cpp_path, py_path = str(tmp_path / "cpp.parquet"), str(tmp_path / "py.parquet")
+    host.save_module(root, cpp_path)
+    table = pq.read_table(cpp_path)
+    assert table.schema.names == ["key", "value"] and str(table.schema.field("key").type) == "string"
+    assert str(table.schema.field("value").type.value_type) == "float"
+    assert pq.ParquetFile(cpp_path).num_row_groups == 1
+    read = ck.load_tensors(cpp_path)
+    assert list(read) == list(before)
+    for k in before:
+        assert torch.equal(read[k], before[k].reshape(-1)), k
+    # the other direction: Python writes other values, C++ loads them into the live module
+    other = {k: torch.randn(v.shape, generator=torch.Generator().manual_seed(i)) for i, (k, v) in enumerate(before.items())}
+    ck.save_tensors(other, py_path)
+    host.load_module(root, py_path)
+    for k, p in root.named_parameters():
+        assert torch.equal(host.to_torch(sched, p).cpu(), other[k]), k
+    # and C++ reads its own file back (test/test_load_save.cpp:86-110)
+    host.load_module(root, cpp_path)
+    for k, p in root.named_parameters():
+        assert torch.equal(host.to_torch(sched, p).cpu(), before[k]), k
+
+
+@pytest.mark.gpu
+def test_cpp_optimizer_checkpoint_resumes_a_run(tmp_path):
+    from core_scheduler_amd import _cs_host as host
+
+    sched = host.DynamicScheduler(0)
+
+    def run(steps, resume_from=None, save_to=None):
+        torch.manual_seed(0)
+        ln = host.LayerNormModule(sched, [32])
+        opt = host.AdamWModule(sched, ln, lr=1e-2, amsgrad=True)
+        if resume_from:
+            host.load_module(ln, resume_from + ".model")
+            host.load_optimizer(opt, resume_from + ".opt")
+        for step in steps:
+            g = torch.Generator().manual_seed(100 + step)
+            x = host.from_torch(sched, torch.randn(8, 32, generator=g).to("cuda:0"))
+            dy = host.from_torch(sched, torch.randn(8, 32, generator=g).to("cuda:0"))
+            ln.forward(sched, x)
+            ln.backward(sched, dy)
+            opt.step(sched)
+            opt.zero_grad(sched)
+        if save_to:
+            host.save_module(ln, save_to + ".model")
+            host.save_optimizer(opt, save_to + ".opt")
+        return ({k: host.to_torch(sched, p).cpu() for k, p in ln.named_parameters()},
+                {k: (host.to_torch(sched, s.m).cpu(), s.t) for k, s in opt.named_states()})
+
+    base = str(tmp_path / "ck")
+    straight, st_straight = run(range(6))
+    run(range(3), save_to=base)
+    rows = ck.load_optimizer(base + ".opt")  # the Python side reads the C++ file
+    assert set(rows) == {"weight", "bias"} and all(r["t"] == 3 and r["v_max"] is not None for r in rows.values())
+    resumed, st_resumed = run(range(3, 6), resume_from=base)
+    for k in straight:
+        assert torch.equal(straight[k], resumed[k]), k
+    for k in st_straight:
+        assert st_straight[k][1] == st_resumed[k][1] == 6
+        assert torch.equal(st_straight[k][0], st_resumed[k][0]), k
