@@ -879,7 +879,17 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
   }
 }
 
-// Standalone position-table gradient (any C, any alignment).
+// Standalone position-table gradient.  The vector form is positions_block on its own (the
+// fused call runs it inside its first launch); the scalar form takes any C and any alignment.
+template <typename T>
+__global__ __launch_bounds__(kTile) void emb_bwd_positions_vec_kernel(const T *__restrict__ dout,
+                                                                      T *__restrict__ dwpe, int64_t B,
+                                                                      int64_t TC, int accumulate,
+                                                                      int log2_slices) {
+  __shared__ f32x4 slices[kPosLdsBytes / sizeof(f32x4)];
+  positions_block<T>(dout, dwpe, blockIdx.x, B, TC, accumulate, log2_slices, slices, threadIdx.x);
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void emb_bwd_positions_kernel(const T *__restrict__ dout,
                                                                      T *__restrict__ dwpe,
@@ -1036,6 +1046,13 @@ int allow_rank_lds(size_t bytes) {
       reinterpret_cast<const void *>(&emb_bwd_rank_kernel<KeyT, IdxT, T>), bytes, done);
 }
 
+// lanes per vector of the position sum: enough that a lane walks at most ~16 rows of the batch
+int position_slices(int64_t B) {
+  int log2_slices = 0;
+  while (log2_slices < kPosMaxLog2Slices && (B >> log2_slices) > 16) ++log2_slices;
+  return log2_slices;
+}
+
 // Sort + merge.  The sort launch also sums dwpe (`fused_positions`), and both launches clear
 // their share of fill_dst[0, fill_vecs), on the CUs the sorting leaves idle.
 template <typename KeyT, typename IdxT, typename T>
@@ -1045,9 +1062,7 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   KeyT *tiles = reinterpret_cast<KeyT *>(ws + L.off_tiles);
   uint32_t *sorted_id = reinterpret_cast<uint32_t *>(ws + L.off_sorted_id);
   uint32_t *sorted_pos = reinterpret_cast<uint32_t *>(ws + L.off_sorted_pos);
-  // lanes per vector of the position sum: enough that a lane walks at most ~16 rows of the batch
-  int pos_log2_slices = 0;
-  while (pos_log2_slices < kPosMaxLog2Slices && (B >> pos_log2_slices) > 16) ++pos_log2_slices;
+  const int pos_log2_slices = position_slices(B);
   const int64_t pos_blocks =
       fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)(kTile >> pos_log2_slices)) : 0;
   const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecs);
@@ -1238,23 +1253,31 @@ extern "C" int cs_embedding_backward_positions(const void *dout, void *dwpe, int
   if (T == 0) return CS_OK;
   if (!dwpe || (B > 0 && !dout)) return CS_ERR_INVALID_ARGUMENT;
   if (!aligned_to(dwpe, es) || (dout && !aligned_to(dout, es))) return CS_ERR_MISALIGNED;
-  int64_t blocks = ceil_div(T * C, (int64_t)kThreads);
-  if (blocks > 65536) blocks = 65536;
   hipStream_t s = as_stream(stream);
-  const dim3 grid((unsigned)blocks), block(kThreads);
+  const int64_t TC = T * C;
+#define CS_POS(T)                                                                                       \
+  do {                                                                                                  \
+    constexpr int VN = Vec16<T>::n;                                                                     \
+    /* an empty batch goes to the scalar kernel, which then writes zeros */                            \
+    if (!std::is_same_v<T, double> && B > 0 && C % VN == 0 && is_aligned16(dout) && is_aligned16(dwpe)) { \
+      const int log2_slices = position_slices(B);                                                       \
+      const int64_t vblocks = ceil_div(TC / VN, (int64_t)(kTile >> log2_slices));                       \
+      if (vblocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;                                              \
+      emb_bwd_positions_vec_kernel<T><<<dim3((unsigned)vblocks), dim3(kTile), 0, s>>>(                  \
+          (const T *)dout, (T *)dwpe, B, TC, accumulate, log2_slices);                                  \
+    } else {                                                                                            \
+      int64_t blocks = ceil_div(TC, (int64_t)kThreads);                                                 \
+      if (blocks > 65536) blocks = 65536;                                                               \
+      emb_bwd_positions_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(                    \
+          (const T *)dout, (T *)dwpe, B, TC, accumulate);                                               \
+    }                                                                                                   \
+  } while (0)
   switch (dtype) {
-    case CS_F32:
-      emb_bwd_positions_kernel<float><<<grid, block, 0, s>>>((const float *)dout, (float *)dwpe, B, T * C, accumulate);
-      break;
-    case CS_F64:
-      emb_bwd_positions_kernel<double><<<grid, block, 0, s>>>((const double *)dout, (double *)dwpe, B, T * C, accumulate);
-      break;
-    case CS_F16:
-      emb_bwd_positions_kernel<f16_t><<<grid, block, 0, s>>>((const f16_t *)dout, (f16_t *)dwpe, B, T * C, accumulate);
-      break;
-    case CS_BF16:
-      emb_bwd_positions_kernel<bf16_t><<<grid, block, 0, s>>>((const bf16_t *)dout, (bf16_t *)dwpe, B, T * C, accumulate);
-      break;
+    case CS_F32: CS_POS(float); break;
+    case CS_F64: CS_POS(double); break;
+    case CS_F16: CS_POS(f16_t); break;
+    case CS_BF16: CS_POS(bf16_t); break;
   }
+#undef CS_POS
   return launch_status();
 }

@@ -65,6 +65,34 @@ def assert_close(got, want, atol, name="", rtol=RTOL):
             f"want {want[i].item()!r}; max abs err {err.max().item():.3e}")
 
 
+def sum_tolerance(terms, dim=0):
+    """Per-output tolerance for fp32 sums over `dim` of `terms`, derived from the data.
+
+    Each of the n - 1 additions rounds its partial sum by at most u = 2^-24 of it; with partial
+    sums of a blocked summation at most ~sqrt(n) rms(terms) and rounding errors of either sign,
+    the error of one sum is ~ u sqrt(log2 n) sqrt(sum terms^2).  Two fp32 evaluations are compared
+    (kernel and oracle) over thousands of outputs, hence the factor 7 (2 x a 3.5 sigma maximum).
+    """
+    t = terms.double()
+    n = max(2, t.shape[dim])
+    return 7.0 * 2.0 ** -24 * torch.sqrt(torch.log2(torch.tensor(float(n))) * (t * t).sum(dim))
+
+
+def assert_sum_close(got, want, tol, name="", rtol=RTOL):
+    """|got - want| <= tol + rtol |want| with a per-element `tol` (see sum_tolerance); 16-bit
+    results may instead be within 1 ulp."""
+    got, want = got.detach().cpu(), want.detach().cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype, name
+    err = (got.double() - want.double()).abs()
+    ok = err <= tol.reshape(want.shape) + rtol * want.double().abs()
+    if got.dtype in (torch.bfloat16, torch.float16):
+        ok |= ulp_distance(got, want) <= 1
+    if not ok.all():
+        i = tuple((~ok).nonzero()[0].tolist())
+        raise AssertionError(f"{name}: {(~ok).sum().item()} of {ok.numel()} sums off; first at {i}: got "
+                             f"{got[i].item()!r} want {want[i].item()!r}, allowed {tol.reshape(want.shape)[i].item():.3e}")
+
+
 def assert_bit_exact(got, want, name=""):
     got, want = got.detach().cpu().contiguous(), want.detach().cpu().contiguous()
     assert got.shape == want.shape and got.dtype == want.dtype, name

@@ -14,7 +14,8 @@ import math
 import pytest
 import torch
 
-from _util import (assert_bit_exact, assert_close, gpt2_param_shapes, randint, randn, zipf_ids)
+from _util import (assert_bit_exact, assert_close, assert_sum_close, gpt2_param_shapes, randint, randn, sum_tolerance,
+                   zipf_ids)
 
 pytestmark = pytest.mark.gpu
 
@@ -300,15 +301,16 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
     dx, dg, db = ops.layernorm_backward(dev(dy), dev(x), dev(mean2), dev(rstd2), dev(gamma), need_dbeta=bias)
     dx2, dg2, db2 = co.layernorm_backward(dy, x, mean2, rstd2, gamma)
     assert_close(dx, dx2, atol=5e-6, name="dx")
-    # column sums of `rows` O(1) terms: the running sum reaches ~sqrt(rows) and each of the
-    # `rows` fp32 additions rounds it by up to 6e-8 of that, so errors add up to the order of
-    # 6e-8 * sqrt(rows) * sqrt(rows); a fifth of that bound is what is allowed here
-    atol_p = 1e-14 if not wide else 1.2e-8 * rows + 1e-6
-    if p_dtype in (torch.bfloat16, torch.float16):
-        atol_p = 1e-6
-    assert_close(dg, dg2, atol=atol_p, name="dgamma")
+    # dgamma and dbeta are column sums over the rows of dy * xhat and dy: the bar is derived from
+    # those terms (see sum_tolerance), not a constant per row
+    if wide:
+        xhat = (x.double() - mean2.double().reshape(-1, 1)) * rstd2.double().reshape(-1, 1)
+        tol_g, tol_b = sum_tolerance(dy.double() * xhat), sum_tolerance(dy)
+    else:
+        tol_g = tol_b = torch.full((C,), 1e-14, dtype=torch.float64)
+    assert_sum_close(dg, dg2, tol_g, name="dgamma")
     if bias:
-        assert_close(db, db2, atol=atol_p, name="dbeta")
+        assert_sum_close(db, db2, tol_b, name="dbeta")
     else:
         assert db is None
 
@@ -593,6 +595,25 @@ def test_embedding_config1(ops, co, kind):
     assert_close(again[0], co.embedding_backward(dout, ids, V, dweight=dwte.cpu()), atol=1e-6, name="dwte +=")
     assert_close(ops.embedding_backward_positions(dev(dout)), co.embedding_backward_positions(dout), atol=1e-6,
                  name="positions alone")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float64])
+@pytest.mark.parametrize("B,T,C", [(1, 8, 64), (8, 128, 768), (16, 64, 1600), (40, 33, 128), (300, 5, 72), (7, 9, 35),
+                                   (0, 4, 64)])
+def test_embedding_positions_alone(ops, co, dtype, B, T, C):
+    """cs_embedding_backward_positions on its own: whole 16-byte vectors take the vector kernel (the batch cut
+    into slices of lanes when it is long), anything else the scalar one; `=` and `+=`; an empty batch gives zeros."""
+    dout = randn((B, T, C), 300 + B + C, dtype=dtype)
+    want = co.embedding_backward_positions(dout) if B > 0 else torch.zeros((T, C), dtype=dtype)
+    got = ops.embedding_backward_positions(dev(dout))
+    # sums over the batch: the bar comes from the terms (fp64 sums are held to 1e-12)
+    tol = sum_tolerance(dout) if dtype != torch.float64 else torch.full((T, C), 1e-12, dtype=torch.float64)
+    assert_sum_close(got, want, tol, name="dwpe")
+    if B > 0:
+        first = got.cpu().clone()
+        ops.embedding_backward_positions(dev(dout), dwpe=got)
+        assert_sum_close(got, co.embedding_backward_positions(dout, dwpe=first), tol, name="dwpe +=")
+        assert_bit_exact(ops.embedding_backward_positions(dev(dout)), ops.embedding_backward_positions(dev(dout)), "rerun")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
