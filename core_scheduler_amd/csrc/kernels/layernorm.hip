@@ -108,6 +108,12 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 #ifndef CS_LN_FWD_PF
 #define CS_LN_FWD_PF true
 #endif
+#ifndef CS_LN_ADD_ROWS_VPL2
+#define CS_LN_ADD_ROWS_VPL2 4
+#endif
+#ifndef CS_LN_ADD_ROWS_VPL4
+#define CS_LN_ADD_ROWS_VPL4 2
+#endif
 constexpr int kLnThreads = 256;  // 4 waves
 // backward launch shape; the defaults are the measured best, the macros exist for tuning runs
 #ifndef CS_LN_BWD_THREADS
@@ -154,11 +160,14 @@ __device__ __forceinline__ void load_rows(RowSet<T, VN, VPL, R> &dst, const T *_
   }
 }
 
-template <typename TX, typename TY, typename TP, int VPL, int R, bool PF>
+// HAS_RES: the rows that are normalised are x + residual, rounded to x's type (the sum is also
+// written to sum_out, which may be x or residual itself): the residual add in front of the
+// LayerNorm of a transformer block without a [rows, C] round trip between two launches.
+template <typename TX, typename TY, typename TP, int VPL, int R, bool PF, bool HAS_RES>
 __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
-    const TX *__restrict__ x, const TP *__restrict__ gamma, const TP *__restrict__ beta,
+    const TX *x /* sum_out may be x: not restrict */, const TP *__restrict__ gamma, const TP *__restrict__ beta,
     TY *__restrict__ y, float *__restrict__ mean, float *__restrict__ rstd, int64_t rows, int C,
-    float eps) {
+    float eps, const TX *res, TX *sum_out) {
   constexpr int VN = Vec16<TX>::n;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t gw = (int64_t)blockIdx.x * (kLnThreads / kWave) + (threadIdx.x >> 6);
@@ -167,8 +176,11 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   int64_t row0 = gw * R;
   if (row0 >= rows) return;  // wave-uniform
 
-  RowSet<TX, VN, VPL, R> cur;
-  if constexpr (PF) load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
+  RowSet<TX, VN, VPL, R> cur, rcur;
+  if constexpr (PF) {
+    load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
+    if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rcur, res, row0, rows, C, nvec, lane);
+  }
   float g[VPL][VN], b[VPL][VN];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
@@ -185,11 +197,31 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   }
   const float inv_c = 1.0f / (float)C;
   for (; row0 < rows; row0 += step) {
-    RowSet<TX, VN, VPL, R> nxt;
+    RowSet<TX, VN, VPL, R> nxt, rnxt;
     if constexpr (PF) {
-      if (row0 + step < rows) load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
+      if (row0 + step < rows) {
+        load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
+        if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rnxt, res, row0 + step, rows, C, nvec, lane);
+      }
     } else {
       load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
+      if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rcur, res, row0, rows, C, nvec, lane);
+    }
+    if constexpr (HAS_RES) {
+      // cur = x + residual, one fp32 add and one rounding per element, as an add launch would give
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          Vec16<TX> sum;
+#pragma unroll
+          for (int k = 0; k < VN; ++k)
+            sum.e[k] = from_acc<TX>(raw_get<TX, VN>(cur.v[r][j], k) + raw_get<TX, VN>(rcur.v[r][j], k));
+          cur.v[r][j].v[0] = sum;
+          const int idx = lane + kWave * j;
+          if (idx < nvec && row0 + r < rows) store16_stream(sum_out + (row0 + r) * C + (int64_t)idx * VN, sum);
+        }
+      }
     }
     // the R rows are independent: their reductions interleave
     float mu[R], rs[R];
@@ -240,7 +272,10 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
         }
       }
     }
-    if constexpr (PF) cur = nxt;
+    if constexpr (PF) {
+      cur = nxt;
+      if constexpr (HAS_RES) rcur = rnxt;
+    }
   }
 }
 
@@ -731,7 +766,7 @@ struct FastPlan {
 };
 // The widest plan whose backward kernel still has registers for a third input per row
 // (dresidual); wider rows get dx + dresidual from a second launch.
-constexpr int kMaxVplWithResidual = 2;
+constexpr int kMaxVplWithResidual = 4;
 
 // x vectors per lane needed for C columns of x_dtype; the fast kernels are
 // instantiated for 2, 4 and 8.
@@ -772,21 +807,32 @@ int ln_blocks(int64_t rows, int rows_per_wave, int cap, int threads = kLnThreads
 
 template <typename TX, typename TY, typename TP>
 int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void *mean, void *rstd,
-              int64_t rows, int64_t C, double eps, bool aligned, int x_dtype, hipStream_t s) {
+              int64_t rows, int64_t C, double eps, bool aligned, int x_dtype, const void *res,
+              void *sum_out, hipStream_t s) {
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
-      const dim3 grid((unsigned)ln_blocks(rows, p.fwd_rows, kLnFwdMaxBlocks)), block(kLnThreads);
-#define CS_LN_FWD(VPL, R)                                                                   \
-  ln_fwd_rows_kernel<TX, TY, TP, VPL, R, CS_LN_FWD_PF><<<grid, block, 0, s>>>(              \
+      // with the residual stream a wave holds two inputs per row: half the rows per step
+      const int r_rows = res ? (p.vpl == 2 ? CS_LN_ADD_ROWS_VPL2 : p.vpl == 4 ? CS_LN_ADD_ROWS_VPL4 : 1) : p.fwd_rows;
+      const dim3 grid((unsigned)ln_blocks(rows, r_rows, kLnFwdMaxBlocks)), block(kLnThreads);
+#define CS_LN_FWD(VPL, R, HAS_RES)                                                          \
+  ln_fwd_rows_kernel<TX, TY, TP, VPL, R, CS_LN_FWD_PF, HAS_RES><<<grid, block, 0, s>>>(     \
       (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean,           \
-      (float *)rstd, rows, (int)C, (float)eps)
-      if (p.vpl == 2) {
-        CS_LN_FWD(2, CS_LN_FWD_ROWS_VPL2);
+      (float *)rstd, rows, (int)C, (float)eps, (const TX *)res, (TX *)sum_out)
+      if (res) {
+        if (p.vpl == 2) {
+          CS_LN_FWD(2, CS_LN_ADD_ROWS_VPL2, true);
+        } else if (p.vpl == 4) {
+          CS_LN_FWD(4, CS_LN_ADD_ROWS_VPL4, true);
+        } else {
+          CS_LN_FWD(8, 1, true);
+        }
+      } else if (p.vpl == 2) {
+        CS_LN_FWD(2, CS_LN_FWD_ROWS_VPL2, false);
       } else if (p.vpl == 4) {
-        CS_LN_FWD(4, CS_LN_FWD_ROWS_VPL4);
+        CS_LN_FWD(4, CS_LN_FWD_ROWS_VPL4, false);
       } else {
-        CS_LN_FWD(8, 1);
+        CS_LN_FWD(8, 1, false);
       }
 #undef CS_LN_FWD
       return launch_status();
@@ -794,6 +840,12 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   }
   using U = typename Acc<TX>::type;
   if (rows > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  if (res) {
+    // no fast plan: the sum as its own launch, then the general kernel on it
+    const int st = launch_add<TX>(x, res, sum_out, rows * C, s);
+    if (st != CS_OK) return st;
+    x = sum_out;
+  }
   ln_fwd_general_kernel<TX, TY, TP><<<dim3((unsigned)rows), dim3(kLnThreads), 0, s>>>(
       (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (U *)mean, (U *)rstd, C,
       (U)eps);
@@ -840,6 +892,10 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
         CS_LN_BWD(2, 3, true, true, true);  // four per SIMD would spill
       } else if (p.vpl == 2 && dres) {
         CS_LN_BWD(2, 4, true, false, true);
+      } else if (p.vpl == 4 && dres && want_dp) {
+        CS_LN_BWD(4, 2, true, true, true);
+      } else if (p.vpl == 4 && dres) {
+        CS_LN_BWD(4, 2, true, false, true);
       } else if (p.vpl == 2) {
         CS_LN_BWD_MASK(2, 4)
       } else if (p.vpl == 4) {
@@ -918,19 +974,12 @@ int ln_forward(const void *x, const void *residual, void *sum_out, const void *g
       (beta && !aligned_to(beta, dtype_size(param_dtype))) || !aligned_to(mean, 4) ||
       !aligned_to(rstd, 4))
     return CS_ERR_MISALIGNED;
-  const bool aligned = is_aligned16(residual ? sum_out : x) && is_aligned16(y) &&
-                       is_aligned16(gamma) && (!beta || is_aligned16(beta));
+  const bool aligned = is_aligned16(x) && (!residual || (is_aligned16(residual) && is_aligned16(sum_out))) &&
+                       is_aligned16(y) && is_aligned16(gamma) && (!beta || is_aligned16(beta));
   hipStream_t s = as_stream(stream);
-  if (residual) {
-    // Measured on MI355X, [8192,768] and [16384,1600] bf16: the sum written by an add launch is
-    // still in the last-level cache when the normalising launch reads it, and the two launches
-    // (17 / 47 us) beat one kernel with two input and two output streams per row (20 / 52 us).
-    const int st = launch_add_dtype(x_dtype, x, residual, sum_out, rows * C, s);
-    if (st != CS_OK) return st;
-    x = sum_out;
-  }
-#define CS_CALL(TX, TY, TP) \
-  return fwd_typed<TX, TY, TP>(x, gamma, beta, y, mean, rstd, rows, C, eps, aligned, x_dtype, s)
+#define CS_CALL(TX, TY, TP)                                                                       \
+  return fwd_typed<TX, TY, TP>(x, gamma, beta, y, mean, rstd, rows, C, eps, aligned, x_dtype, residual, \
+                               sum_out, s)
   const bool y_wide = y_dtype != x_dtype, p_wide = param_dtype != x_dtype;
   switch (x_dtype) {
     case CS_F32: CS_CALL(float, float, float);
