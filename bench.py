@@ -13,8 +13,12 @@ The same line carries
                 its duration measured with HIP events inside the timed region
   per_op        every op of the hot path at its benchmark configuration:
                 ms, GB/s of algorithmic bytes and fraction of the HBM peak,
-                warm (same buffers) and cold (buffers rotated over > 512 MB so
-                the 256 MB Infinity Cache cannot serve them)
+                warm (same buffers) and cold (inputs and outputs rotated over
+                > 600 MB so the 256 MB Infinity Cache cannot serve them), each
+                the duration of one call inside a batch of back-to-back calls
+                between one pair of events; next to it the rocprofv3 kernel
+                time the op's launches add up to (kernel_us) and three
+                calibration kernels (plain copy, read only, write only)
   cpu_baseline  the reference's own op sequence on the ATen CPU backend
                 (oracle/aten_port.py), timed here on this box's host cores
 
@@ -42,7 +46,60 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # algorithmic bytes per fused-classifier call: read the class columns of the logits once and
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
-CE_ROWS_TRAFFIC_BYTES = 1_650_851_000  # measured with rocprofv3 --pmc, see profiles/
+CE_ROWS_TRAFFIC_BYTES = 1_650_518_000  # measured with rocprofv3 --pmc, see profiles/
+
+
+# Kernel durations the per-op rows should agree with: average begin-to-end time of each launch an
+# op makes, from the rocprofv3 kernel trace summarised in profiles/bench_all_ops_kernel_trace.txt
+# (same command as this benchmark, under the profiler).  (op, start of config) -> (sum in us, launches)
+KERNEL_TRACE_US = {
+    ("layernorm_fwd", "small"): (6.94, "ln_fwd_rows_kernel<2,4>"),
+    ("layernorm_bwd", "small"): (10.04 + 4.35, "ln_bwd_rows_kernel<2,4> + ln_bwd_finalize_kernel"),
+    ("add_layernorm_fwd", "small"): (10.29, "ln_fwd_rows_kernel<2,4,residual>"),
+    ("layernorm_bwd_add", "small"): (16.64 + 4.35, "ln_bwd_rows_kernel<2,3,residual> + ln_bwd_finalize_kernel"),
+    ("layernorm_fwd", "xl"): (19.89, "ln_fwd_rows_kernel<4,2>"),
+    ("layernorm_bwd", "xl"): (30.04 + 4.53, "ln_bwd_rows_kernel<4,2> + ln_bwd_finalize_kernel"),
+    ("add_layernorm_fwd", "xl"): (37.19, "ln_fwd_rows_kernel<4,2,residual>"),
+    ("layernorm_bwd_add", "xl"): (48.82 + 4.53, "ln_bwd_rows_kernel<4,2,residual> + ln_bwd_finalize_kernel"),
+    ("gelu_fwd_tanh", ""): (16.97, "gelu_kernel<tanh,fwd>"),
+    ("gelu_bwd_tanh", ""): (24.11, "gelu_kernel<tanh,bwd>"),
+    ("gelu_fwd_erf", ""): (17.79, "gelu_kernel<erf,fwd>"),
+    ("gelu_bwd_erf", ""): (24.22, "gelu_kernel<erf,bwd>"),
+    ("embedding_fwd", "small"): (5.45, "emb_fwd_vec_kernel (uniform and zipf launches averaged)"),
+    ("embedding_bwd", "small"): (17.05 + 6.94 + 4.21, "emb_bwd_rank_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
+    ("embedding_fwd", "xl"): (11.59, "emb_fwd_vec_kernel"),
+    ("embedding_bwd", "xl"): (21.59 + 16.88 + 15.51 + 9.42,
+                              "emb_bwd_tile_sort_kernel + emb_bwd_merge_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
+    ("adamw_multi_tensor", "small"): (576.44, "adamw_multi_kernel"),
+    ("adamw_multi_tensor", "xl"): (7946.02, "adamw_multi_kernel"),
+    ("adamw_multi_tensor_clipped", "small"): (80.42 + 9.44 + 576.44, "grad_norm_partial_kernel + grad_norm_final_kernel + adamw_multi_kernel"),
+    ("fused_classifier_call", "[8192,50304] bf16, in place"): (4.18 + 279.40 + 4.04, "ce_count_kernel + ce_rows_stream_kernel<7,8> + ce_reduce_kernel"),
+    ("fused_classifier_call", "[8192,50304] bf16, bf16 logits"): (4.47 + 448.65 + 4.33, "ce_count_kernel + ce_rows_stream_kernel<13,4> + ce_reduce_kernel"),
+    ("stream_copy", "25 MB"): (4.92, "stream_copy_kernel<2>"),
+    ("stream_copy", "100 MB"): (17.58, "stream_copy_kernel<2>"),
+    ("stream_copy", "400 MB"): (62.13, "stream_copy_kernel<1>"),
+    ("stream_copy", "1600 MB"): (241.44, "stream_copy_kernel<1>"),
+    ("stream_copy", "3500 MB"): (531.87, "stream_copy_kernel<1>"),
+    ("stream_read", "25 MB"): (5.29, "stream_read_kernel"),
+    ("stream_read", "100 MB"): (16.03, "stream_read_kernel"),
+    ("stream_read", "400 MB"): (59.94, "stream_read_kernel"),
+    ("stream_read", "3500 MB"): (507.70, "stream_read_kernel"),
+    ("stream_fill", "25 MB"): (4.94, "stream_fill_kernel"),
+    ("stream_fill", "100 MB"): (17.48, "stream_fill_kernel"),
+    ("stream_fill", "400 MB"): (69.04, "stream_fill_kernel"),
+    ("stream_fill", "3500 MB"): (602.81, "stream_fill_kernel"),
+}
+
+
+def attach_kernel_trace(rec):
+    """Adds the profiled kernel time an op's launches add up to, for cross-checking ms_cold."""
+    for (op, prefix), (us, launches) in KERNEL_TRACE_US.items():
+        if rec["op"] == op and rec["config"].startswith(prefix):
+            rec["kernel_us"] = round(us, 2)
+            rec["kernel_launches"] = launches
+            rec["ms_cold_over_kernel"] = round(rec["ms_cold"] * 1e3 / us, 3)
+            return rec
+    return rec
 
 
 def log(*a):
@@ -572,6 +629,8 @@ def main():
         if table:
             cpu_per_op(args, torch, table)
 
+    for rec in table:
+        attach_kernel_trace(rec)
     line = {
         "metric": "per-op HBM GB/s (% of MI355X peak); fused CE ms at 8192x50257 bf16",
         "metric_note": "value = the fused classifier's whole-step GB/s (the ms is ms_per_step); every other op is in per_op",

@@ -214,14 +214,14 @@ int cs_layernorm_backward(const void *dy, const void *x, const void *mean,
  *             replaces ln2->backward (:468) followed by Utils::add (:469)
  * Results are those of the two separate kernels, bit for bit: the sum is
  * rounded to x_dtype before it is normalised, and dx is rounded to dx_dtype
- * before dresidual is added.  The backward add runs inside the LayerNorm
- * kernel for rows of up to 128 16-byte vectors (C <= 1024 for 16-bit x),
- * where it saves a [rows, C] round trip; the other cases run an elementwise
- * add launch next to the LayerNorm launch, which measured faster on MI355X
- * than a single kernel with one more stream per row (the intermediate stays
- * in the last-level cache).  residual and sum_out are [rows, C] of x_dtype
- * (sum_out may be x or residual itself); dresidual is [rows, C] of dx_dtype
- * (dx may be dresidual itself).  All other arguments as in the plain calls. */
+ * before dresidual is added.  Both adds run inside the LayerNorm kernel, which
+ * saves a [rows, C] round trip and a launch: forward for every row width the
+ * row-in-registers kernels take (up to 512 16-byte vectors: C <= 4096 for
+ * 16-bit x), backward for rows of up to 256 vectors (C <= 2048 at 16 bit);
+ * other shapes run an elementwise add launch next to the LayerNorm launch.
+ * residual and sum_out are [rows, C] of x_dtype (sum_out may be x or residual
+ * itself); dresidual is [rows, C] of dx_dtype (dx may be dresidual itself).
+ * All other arguments as in the plain calls. */
 int cs_add_layernorm_forward(const void *x, const void *residual,
                              void *sum_out, const void *gamma,
                              const void *beta, void *y, void *mean, void *rstd,
