@@ -342,6 +342,29 @@ def per_op_table(args, torch, ops):
         add("layernorm_bwd", f"{tag} [{rows},{C}] bf16", bwd_bytes, mk,
             lambda s: ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma))
 
+        # the reference's schedule: input gradient on the main stream, parameter gradients on the
+        # assist stream.  The timed stream runs the row pass; a second stream adds the partial rows
+        # up, and the timed stream waits for that two calls later, as the host scheduler does
+        side = torch.cuda.Stream(dev)
+        pending = []
+
+        def two_streams(s):
+            main = torch.cuda.current_stream(dev)
+            if len(pending) >= 2:
+                main.wait_event(pending.pop(0))
+            dx, partials = ops.layernorm_backward_rows(s["dy"], s["x"], s["mean"], s["rstd"], gamma)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                dg, db = ops.layernorm_backward_finalize(partials, torch.bfloat16, torch.float32)
+                done = torch.cuda.Event()
+                done.record(side)
+            partials.record_stream(side)
+            pending.append(done)
+            return dx, dg, db
+
+        add("layernorm_bwd_two_streams", f"{tag} [{rows},{C}] bf16, row pass timed, sums on a second stream",
+            bwd_bytes, mk, two_streams)
+
         # the residual stream folded into the call (x + residual -> LayerNorm; LayerNorm backward
         # + dresidual), next to the same work as a separate elementwise add around the plain call
         def mk_res():

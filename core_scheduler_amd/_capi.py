@@ -79,6 +79,15 @@ SIGNATURES = {
         [c_void_p] * 10 + [c_size_t, c_int64, c_int64] + [c_int] * 5 + [c_void_p],
     ),
     "cs_layernorm_backward_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "cs_layernorm_backward_partial_rows": (c_int64, [c_int64, c_int64, c_int]),
+    "cs_layernorm_backward_rows": (
+        c_int,
+        [c_void_p] * 8 + [c_size_t, c_int64, c_int64] + [c_int] * 4 + [c_void_p],
+    ),
+    "cs_layernorm_backward_finalize": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
+    ),
     "cs_layernorm_backward": (
         c_int,
         [c_void_p] * 9 + [c_size_t, c_int64, c_int64] + [c_int] * 5 + [c_void_p],

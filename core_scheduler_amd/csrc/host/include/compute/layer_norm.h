@@ -64,7 +64,8 @@ struct CS_API LayerNorm {
 
   // One task on the main stream producing dx, dgamma and dbeta from a single pass over dy
   // and x (the reference submits a parameter task on the assist stream and an input task on
-  // the main stream, each a full native_layer_norm_backward call).
+  // the main stream, each a full native_layer_norm_backward call; the second stream costs the
+  // main stream more in waiting than the 4 us of summing it would take over).
   static Tensor backward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
                          const ReadOnlyTensor &grad_output);
 };

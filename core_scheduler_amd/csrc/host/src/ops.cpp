@@ -101,8 +101,12 @@ Tensor CrossEntropy::forward(const Scheduler &scheduler, const std::shared_ptr<S
                                 dtype_of(x.scalar_type()), dtype_of(g_type), current_stream()),
             name());
       T(output()[0]) = grad;
-      T(output()[1]) = args.reduction == at::Reduction::None ? rows : loss;
-      T(output()[2]) = total;
+      // The reference hands out what nll_loss_forward returns: loss and total weight in the dtype
+      // of the log-probabilities (cross_entropy.cpp:57-66), which is 16-bit for 16-bit logits
+      // outside autocast.  The kernel sums in fp32; the rounding to that dtype happens once, here.
+      const at::Tensor &result = args.reduction == at::Reduction::None ? rows : loss;
+      T(output()[1]) = g_type == at::kFloat ? result : result.to(g_type);
+      T(output()[2]) = g_type == at::kFloat ? total : total.to(g_type);
     }
     [[nodiscard]] const char *name() const override { return "cs::compute::CrossEntropy::forward"; }
   };
@@ -463,6 +467,11 @@ Tensor LayerNorm::forward(const Scheduler &scheduler, const std::shared_ptr<Stat
 
 Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
                            const ReadOnlyTensor &grad_output) {
+  // One task on the main stream.  The reference submits two (parameter gradients on the assist
+  // stream, src/compute/layer_norm.cpp:228-233), and the kernels can be called that way
+  // (cs_layernorm_backward_rows / _finalize), but the second kernel is 4 us of work, while making
+  // the main stream wait for another stream's event costs it 7 us on this part: at [8192, 768]
+  // the main stream is busy 13.9 us per call with one task and 18.8 us with two.
   struct Body final : Task::Impl {
     bool has_bias;
     Body(std::vector<Tensor> out /* dx, grad_weight[, grad_bias] */,

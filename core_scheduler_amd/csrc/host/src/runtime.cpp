@@ -35,7 +35,10 @@ struct Event::Impl {
   void synchronize() const { event.synchronize(); }
 
  private:
-  at::cuda::CUDAEvent event;
+  // Events here order streams of one device and tell the host that work has finished; the data
+  // itself reaches the host through stream-ordered copies.  Without the system-scope fence a
+  // record costs the stream 0.9 us instead of 2.7 us (measured behind a 14 us kernel).
+  at::cuda::CUDAEvent event{hipEventDisableTiming | hipEventDisableSystemFence};
 };
 
 namespace {
@@ -140,23 +143,29 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
       try {
         age(assist_);
         age(comm_);
-        run(task, lane);
-        main_done_.record();
+        replace(main_done_, run(task, lane));
       } catch (const std::exception &e) {
         CS_ASSERT_TRUE(false, std::string("Task ") + body.name() + " failed with error: " + e.what());
       }
       return;
     }
     main_done_.block();
-    run(task, lane);
-    Parked parked{lane == Priority::kAssist ? kAssistGap : kCommGap, Event{}, touched(body)};
-    parked.done.record();
+    Parked parked{lane == Priority::kAssist ? kAssistGap : kCommGap, run(task, lane), touched(body)};
     (lane == Priority::kAssist ? assist_ : comm_).push_front(std::move(parked));
   }
 
  private:
-  // make the current stream wait for inputs from other streams, run, stamp the outputs
-  static void run(const Task &task, const Priority lane) {
+  // `slot` becomes another handle of `stamp`; the event it held goes back to the pool if this
+  // was its last handle
+  static void replace(Event &slot, const Event &stamp) {
+    const Event old{slot};
+    slot = stamp;
+  }
+  // Make the current stream wait for inputs from other streams, run, stamp the outputs.  One
+  // event is recorded per task (the reference records one per output tensor,
+  // src/threading/dynamic_scheduler.cpp:150-160): every output, and the caller's own
+  // bookkeeping, share it, since each record is a packet the stream has to work through.
+  static Event run(const Task &task, const Priority lane) {
     for (const auto &t : task.impl()->input()) {
       if (t.impl()->priority() != lane && !t.impl()->event().query()) t.impl()->event().block();
     }
@@ -165,16 +174,20 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
       const TraceRange range{task.impl()->name()};
       task();
     }
+    Event stamp;
+    stamp.record();
     for (const auto &t : task.impl()->output()) {
       t.impl()->priority() = lane;
-      t.impl()->event().record();
+      replace(t.impl()->event(), stamp);
     }
+    return stamp;
   }
-  // one more main task has arrived: side-stream work that is old enough is waited for
+  // one more main task has arrived: side-stream work that is old enough is waited for, unless
+  // it has finished already (a wait costs the main stream about 7 us even then)
   static void age(std::deque<Parked> &queue) {
     for (auto &p : queue) --p.countdown;
     while (!queue.empty() && queue.back().countdown <= 0) {
-      queue.back().done.block();
+      if (!queue.back().done.query()) queue.back().done.block();
       queue.pop_back();
     }
   }

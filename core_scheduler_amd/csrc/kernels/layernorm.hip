@@ -852,13 +852,26 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   return launch_status();
 }
 
+// Partial rows [2C fp32 each] that the row kernel of a plan leaves for the finalize kernel.
+int bwd_partial_rows(int64_t rows, int vpl) {
+  // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
+  if (vpl == 8) return ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
+  return ln_blocks(rows, 1, vpl == 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
+}
+
+enum BwdPhase { kBwdWhole = 0, kBwdRowsOnly = 1 };
+
 template <typename TDY, typename TX, typename TDX, typename TP>
 int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
               const void *gamma, void *dx, void *dgamma, void *dbeta, void *workspace,
               size_t workspace_bytes, int64_t rows, int64_t C, bool aligned, int x_dtype,
-              int accumulate, const void *dres, hipStream_t s) {
-  const bool want_dp = dgamma != nullptr || dbeta != nullptr;
+              int accumulate, const void *dres, hipStream_t s, BwdPhase phase = kBwdWhole) {
+  // rows only: the partial rows are the product, the parameter gradients come from a later
+  // cs_layernorm_backward_finalize
+  const bool want_dp = phase == kBwdRowsOnly || dgamma != nullptr || dbeta != nullptr;
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
+  if (phase == kBwdRowsOnly && (p.vpl == 0 || std::is_same_v<TX, double>))
+    return aligned ? CS_ERR_UNSUPPORTED : CS_ERR_MISALIGNED;
   // dx + dresidual inside the kernel where it fits (17.5 -> 22 us against 25 us for two
   // launches at [8192,768] bf16), as a second, in-place launch elsewhere
   const bool fuse_dres = dres != nullptr && p.vpl != 0 && p.vpl <= kMaxVplWithResidual && is_aligned16(dres);
@@ -868,9 +881,8 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
     if (p.vpl != 0) {
       const int blocks =
           ln_blocks(rows, 1, p.vpl == 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
-      // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
-      const int split_blocks = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
-      int blocks_used = p.vpl == 8 && want_dp ? split_blocks : blocks;  // partial rows left behind
+      const int split_blocks = bwd_partial_rows(rows, 8);
+      const int blocks_used = want_dp ? bwd_partial_rows(rows, p.vpl) : blocks;  // partial rows left behind
       const size_t need = want_dp ? (size_t)blocks_used * 2 * C * sizeof(float) : 0;
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
       const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
@@ -920,7 +932,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
 #undef CS_LN_BWD_MASK
 #undef CS_LN_BWD
       int st = launch_status();
-      if (st == CS_OK && want_dp) {
+      if (st == CS_OK && want_dp && phase == kBwdWhole) {
         ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)kLnFinCols), 2), dim3(kLnFinCols, kLnFinRows), 0, s>>>(
             (const float *)workspace, blocks_used, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
         st = launch_status();
@@ -1028,7 +1040,8 @@ namespace {
 int ln_backward(const void *dy, const void *x, const void *mean, const void *rstd,
                 const void *gamma, const void *dres, void *dx, void *dgamma, void *dbeta,
                 void *workspace, size_t workspace_bytes, int64_t rows, int64_t C, int dy_dtype,
-                int x_dtype, int dx_dtype, int param_dtype, int accumulate, void *stream) {
+                int x_dtype, int dx_dtype, int param_dtype, int accumulate, void *stream,
+                BwdPhase phase = kBwdWhole) {
   if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
   if (dtype_size(x_dtype) == 0 || dtype_size(dy_dtype) == 0 || dtype_size(dx_dtype) == 0 ||
       dtype_size(param_dtype) == 0)
@@ -1037,7 +1050,7 @@ int ln_backward(const void *dy, const void *x, const void *mean, const void *rst
     return CS_ERR_UNSUPPORTED;
   if (x_dtype == CS_F64 && (dy_dtype != CS_F64 || dx_dtype != CS_F64 || param_dtype != CS_F64))
     return CS_ERR_UNSUPPORTED;
-  if (!dx && !dgamma && !dbeta) return CS_OK;
+  if (phase == kBwdWhole && !dx && !dgamma && !dbeta) return CS_OK;
   if (rows == 0) {
     // an empty batch still defines dgamma/dbeta: zero unless accumulating;
     // nothing to launch for that without rows, so leave it to the caller
@@ -1059,7 +1072,7 @@ int ln_backward(const void *dy, const void *x, const void *mean, const void *rst
   hipStream_t s = as_stream(stream);
 #define CS_CALL(TDY, TX, TDX, TP)                                                              \
   return bwd_typed<TDY, TX, TDX, TP>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, workspace,   \
-                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, dres, s)
+                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, dres, s, phase)
   const bool dy_wide = dy_dtype != x_dtype, dx_wide = dx_dtype != x_dtype,
              p_wide = param_dtype != x_dtype;
   switch (x_dtype) {
@@ -1102,4 +1115,52 @@ extern "C" int cs_layernorm_backward_add(const void *dy, const void *x, const vo
   return ln_backward(dy, x, mean, rstd, gamma, dresidual, dx, dgamma, dbeta, workspace,
                      workspace_bytes, rows, C, dy_dtype, x_dtype, dx_dtype, param_dtype, accumulate,
                      stream);
+}
+
+extern "C" int64_t cs_layernorm_backward_partial_rows(int64_t rows, int64_t C, int x_dtype) {
+  if (rows <= 0 || C <= 0 || dtype_size(x_dtype) == 0) return 0;
+  const FastPlan p = fast_plan(C, x_dtype);
+  return p.vpl == 0 ? 0 : bwd_partial_rows(rows, p.vpl);
+}
+
+extern "C" int cs_layernorm_backward_rows(const void *dy, const void *x, const void *mean,
+                                          const void *rstd, const void *gamma,
+                                          const void *dresidual, void *dx, void *partials,
+                                          size_t partials_bytes, int64_t rows, int64_t C,
+                                          int dy_dtype, int x_dtype, int dx_dtype,
+                                          int param_dtype, void *stream) {
+  if (rows <= 0 || C <= 0 || !partials || !gamma) return CS_ERR_INVALID_ARGUMENT;
+  if (dresidual && !dx) return CS_ERR_INVALID_ARGUMENT;
+  return ln_backward(dy, x, mean, rstd, gamma, dresidual, dx, nullptr, nullptr, partials,
+                     partials_bytes, rows, C, dy_dtype, x_dtype, dx_dtype, param_dtype, 0, stream,
+                     kBwdRowsOnly);
+}
+
+extern "C" int cs_layernorm_backward_finalize(const void *partials, int64_t partial_rows,
+                                              void *dgamma, void *dbeta, int64_t C, int x_dtype,
+                                              int param_dtype, int accumulate, void *stream) {
+  if (C <= 0 || partial_rows <= 0 || !partials) return CS_ERR_INVALID_ARGUMENT;
+  if (dtype_size(x_dtype) == 0 || dtype_size(param_dtype) == 0 || x_dtype == CS_F64 ||
+      !wide_ok(x_dtype, param_dtype))
+    return CS_ERR_UNSUPPORTED;
+  const int vn = 16 / (int)dtype_size(x_dtype);
+  if (C % vn != 0 || partial_rows > (kLnBwdMaxBlocksNarrow > kLnBwdMaxBlocks ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks))
+    return CS_ERR_INVALID_ARGUMENT;
+  if (!dgamma && !dbeta) return CS_OK;
+  if (!is_aligned16(partials) || (dgamma && !aligned_to(dgamma, dtype_size(param_dtype))) ||
+      (dbeta && !aligned_to(dbeta, dtype_size(param_dtype))))
+    return CS_ERR_MISALIGNED;
+  hipStream_t s = as_stream(stream);
+  const dim3 grid((unsigned)ceil_div(C, (int64_t)kLnFinCols), 2), block(kLnFinCols, kLnFinRows);
+#define CS_FIN(TP)                                                                              \
+  ln_bwd_finalize_kernel<TP><<<grid, block, 0, s>>>((const float *)partials, (int)partial_rows, \
+                                                    (TP *)dgamma, (TP *)dbeta, (int)C, vn, accumulate)
+  switch (param_dtype) {
+    case CS_F32: CS_FIN(float); break;
+    case CS_F16: CS_FIN(f16_t); break;
+    case CS_BF16: CS_FIN(bf16_t); break;
+    default: return CS_ERR_UNSUPPORTED;
+  }
+#undef CS_FIN
+  return launch_status();
 }

@@ -285,10 +285,68 @@ def layernorm_backward(dy, x, mean, rstd, gamma, *, need_dx=True, need_dgamma=Tr
         else:
             code = lib.cs_layernorm_backward(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma), _ptr(dx),
                                              _ptr(dgamma), _ptr(dbeta), _ptr(ws), ws_bytes, rows, C, _dt(dy),
-                                             _dt(x), _dt(dx) if dx is not None else _dt(x), _dt(gamma),
+                                             _dt(x), _dt(dx) if dx is not None else _dt(dy), _dt(gamma),
                                              int(accumulate), _stream(dev))
     _capi.check("cs_layernorm_backward", code)
     return dx, dgamma, dbeta
+
+
+def layernorm_backward_rows(dy, x, mean, rstd, gamma, *, need_dx=True, dx_dtype=None, dresidual=None):
+    """First half of the backward pass as two tasks (main stream): returns (dx, partials).
+
+    `partials` is a new fp32 tensor [partial_rows, 2, C] for `layernorm_backward_finalize`, which
+    may run on another stream once this call's work is done.  Raises ValueError for shapes that
+    have no split form (use `layernorm_backward`).
+    """
+    dev = _dev(dy, x, mean, rstd, gamma, dresidual)
+    if dresidual is not None and (not need_dx or dresidual.shape != x.shape
+                                  or dresidual.dtype != (dx_dtype or x.dtype)):
+        raise ValueError("dresidual must match dx")
+    C = x.shape[-1]
+    rows = x.numel() // C
+    lib = _capi.load()
+    n = lib.cs_layernorm_backward_partial_rows(rows, C, _dt(x))
+    if n == 0:
+        raise ValueError(f"no split form for rows of {C} {x.dtype} elements")
+    dx = torch.empty(x.shape, dtype=dx_dtype or x.dtype, device=dev) if need_dx else None
+    partials = torch.empty((n, 2, C), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        code = lib.cs_layernorm_backward_rows(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma),
+                                              _ptr(dresidual), _ptr(dx), _ptr(partials), partials.numel() * 4,
+                                              rows, C, _dt(dy), _dt(x), _dt(dx) if dx is not None else _dt(dy),
+                                              _dt(gamma), _stream(dev))
+    _capi.check("cs_layernorm_backward_rows", code)
+    return dx, partials
+
+
+def layernorm_backward_finalize(partials, x_dtype, param_dtype, *, need_dgamma=True, need_dbeta=True,
+                                dgamma=None, dbeta=None):
+    """Second half: (dgamma, dbeta) from the partial rows, added in a fixed order.  Passing
+    dgamma / dbeta accumulates into them.  `x_dtype` is the dtype of the x the rows call read."""
+    dev = _dev(partials, dgamma, dbeta)
+    n, two, C = partials.shape
+    if two != 2 or partials.dtype != torch.float32 or not partials.is_contiguous():
+        raise ValueError("partials must be the contiguous fp32 [n, 2, C] tensor of layernorm_backward_rows")
+    accumulate = dgamma is not None or dbeta is not None
+    if accumulate and ((need_dgamma and dgamma is None) or (need_dbeta and dbeta is None)):
+        raise ValueError("accumulating needs every requested parameter gradient passed in")
+    for g in (dgamma, dbeta):
+        if g is not None and (g.dtype != param_dtype or g.numel() != C):
+            raise ValueError("dgamma / dbeta must be [C] of the parameter dtype")
+    if need_dgamma and dgamma is None:
+        dgamma = torch.empty(C, dtype=param_dtype, device=dev)
+    if need_dbeta and dbeta is None:
+        dbeta = torch.empty(C, dtype=param_dtype, device=dev)
+    if not need_dgamma:
+        dgamma = None
+    if not need_dbeta:
+        dbeta = None
+    with torch.cuda.device(dev):
+        code = _capi.load().cs_layernorm_backward_finalize(_ptr(partials), n, _ptr(dgamma), _ptr(dbeta), C,
+                                                           _DTYPES[x_dtype], _DTYPES[param_dtype], int(accumulate),
+                                                           _stream(dev))
+    _capi.check("cs_layernorm_backward_finalize", code)
+    return dgamma, dbeta
 
 
 # -------------------------------------------------------------- Embedding

@@ -235,6 +235,37 @@ int cs_layernorm_backward_add(const void *dy, const void *x, const void *mean,
                               int dy_dtype, int x_dtype, int dx_dtype,
                               int param_dtype, int accumulate, void *stream);
 
+/* LayerNorm backward as the reference schedules it: the input gradient is a
+ * task on the main stream (src/compute/layer_norm.cpp:235-283, kMain), the
+ * parameter gradients a task on the assist stream (:285-400, kAssist).  Here
+ * the first task reads dy and x once and leaves, next to dx, per-workgroup
+ * column sums of dy*xhat and dy ("partial rows", fp32 [partial_rows, 2, C]);
+ * the second adds those rows in a fixed order, which is a few hundred KB of
+ * work and can run on another stream while the main stream goes on.  The pair
+ * gives the bits of cs_layernorm_backward (same kernels, same order).
+ *
+ * cs_layernorm_backward_partial_rows: rows of the partial buffer for this
+ *   shape (the buffer holds partial_rows * 2 * C floats), or 0 when the shape
+ *   has no split form (C not a multiple of the 16-byte vector, rows wider than
+ *   512 vectors, CS_F64): use cs_layernorm_backward then.
+ * cs_layernorm_backward_rows: dx (may be NULL) and the partial rows;
+ *   dresidual as in cs_layernorm_backward_add or NULL.  All pointers 16-byte
+ *   aligned (CS_ERR_MISALIGNED otherwise).
+ * cs_layernorm_backward_finalize: dgamma / dbeta (either may be NULL) from the
+ *   partial rows; x_dtype is the one the rows call was given (it fixes the
+ *   column order inside a partial row). */
+int64_t cs_layernorm_backward_partial_rows(int64_t rows, int64_t C, int x_dtype);
+int cs_layernorm_backward_rows(const void *dy, const void *x, const void *mean,
+                               const void *rstd, const void *gamma,
+                               const void *dresidual, void *dx, void *partials,
+                               size_t partials_bytes, int64_t rows, int64_t C,
+                               int dy_dtype, int x_dtype, int dx_dtype,
+                               int param_dtype, void *stream);
+int cs_layernorm_backward_finalize(const void *partials, int64_t partial_rows,
+                                   void *dgamma, void *dbeta, int64_t C,
+                                   int x_dtype, int param_dtype, int accumulate,
+                                   void *stream);
+
 /* ------------------------------------------------------------------------
  * Embedding
  * forward replaces torch::embedding, src/compute/embedding.cpp:117-121:

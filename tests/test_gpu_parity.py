@@ -468,6 +468,63 @@ def test_layernorm_masks_and_accumulate(ops, co):
         assert_bit_exact(a, b, "rerun")
 
 
+@pytest.mark.parametrize("rows,C,x_dtype,p_dtype,wide_dy", [
+    (8192, 768, torch.bfloat16, torch.float32, False),    # benchmark configuration 3
+    (700, 768, torch.bfloat16, torch.float32, True),      # the autocast combination: fp32 dy and dx
+    (2048, 1600, torch.bfloat16, torch.float32, False),   # XL width
+    (513, 768, torch.float16, torch.float16, False),
+    (77, 4096, torch.bfloat16, torch.float32, False),     # two waves per row
+    (2051, 1600, torch.float32, torch.float32, False),
+    (3, 768, torch.float32, torch.float32, False),
+])
+def test_layernorm_backward_as_two_calls(ops, rows, C, x_dtype, p_dtype, wide_dy):
+    """Row pass on one stream, sum of the partial rows on another (the reference's main and
+    assist tasks, src/compute/layer_norm.cpp:228-233): the bits of the single call."""
+    x = randn((rows, C), 80, dtype=x_dtype)
+    gamma = randn(C, 81, std=0.02, mean=1.0, dtype=p_dtype)
+    dy = randn((rows, C), 82, dtype=torch.float32 if wide_dy else x_dtype)
+    mean = x.float().mean(-1)
+    rstd = 1.0 / torch.sqrt(x.float().var(-1, unbiased=False) + 1e-5)
+    res = randn((rows, C), 83, dtype=dy.dtype)
+    gx, gdy, gm, gr, gg, gres = dev(x), dev(dy), dev(mean), dev(rstd), dev(gamma), dev(res)
+    whole = ops.layernorm_backward(gdy, gx, gm, gr, gg, dx_dtype=dy.dtype)
+    side = torch.cuda.Stream()
+    dx, partials = ops.layernorm_backward_rows(gdy, gx, gm, gr, gg, dx_dtype=dy.dtype)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        dg, db = ops.layernorm_backward_finalize(partials, x_dtype, p_dtype)
+    side.synchronize()
+    assert_bit_exact(dx, whole[0], "dx")
+    assert_bit_exact(dg, whole[1], "dgamma")
+    assert_bit_exact(db, whole[2], "dbeta")
+    # dgamma only, += into an existing gradient, and dresidual in the row pass
+    dg0 = randn(C, 84, dtype=p_dtype)
+    acc_whole = dev(dg0)
+    ops.layernorm_backward(gdy, gx, gm, gr, gg, need_dx=False, need_dbeta=False, dgamma=acc_whole)
+    acc = dev(dg0)
+    got = ops.layernorm_backward_finalize(partials, x_dtype, p_dtype, need_dbeta=False, dgamma=acc)
+    assert got[1] is None and got[0] is acc
+    assert_bit_exact(acc, acc_whole, "dgamma +=")
+    with_res = ops.layernorm_backward(gdy, gx, gm, gr, gg, dx_dtype=dy.dtype, dresidual=gres)
+    dx_r, partials_r = ops.layernorm_backward_rows(gdy, gx, gm, gr, gg, dx_dtype=dy.dtype, dresidual=gres)
+    assert_bit_exact(dx_r, with_res[0], "dx + dresidual")
+    assert_bit_exact(ops.layernorm_backward_finalize(partials_r, x_dtype, p_dtype)[0], with_res[1], "dgamma, residual form")
+    # no dx: the parameter half on its own
+    none_dx, partials_p = ops.layernorm_backward_rows(gdy, gx, gm, gr, gg, need_dx=False)
+    assert none_dx is None
+    assert_bit_exact(ops.layernorm_backward_finalize(partials_p, x_dtype, p_dtype)[1], whole[2], "dbeta without dx")
+
+
+def test_layernorm_backward_shapes_without_two_call_form(ops):
+    lib = __import__("core_scheduler_amd._capi", fromlist=["load"]).load()
+    assert lib.cs_layernorm_backward_partial_rows(64, 50, 0) == 0       # C not a multiple of the vector
+    assert lib.cs_layernorm_backward_partial_rows(64, 10000, 3) == 0    # wider than the register plans
+    assert lib.cs_layernorm_backward_partial_rows(0, 768, 3) == 0
+    x = dev(randn((64, 50), 85))
+    with pytest.raises(ValueError):
+        ops.layernorm_backward_rows(x, x, dev(randn(64, 86)), dev(randn(64, 87)), dev(randn(50, 88)))
+
+
 # -------------------------------------------------------------- Embedding
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("idx_dtype", [torch.int32, torch.int64])

@@ -176,9 +176,14 @@ def test_cross_entropy_amp(host, sched, co, dtype):
     assert_close(got, want_dx, atol=1e-9, name="dx fp32")
     # outside the guard the gradient keeps the logits' dtype; padded vocabulary via num_classes
     state = host.CrossEntropy.init(sched, num_classes=300)
-    host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t % 300))
+    loss16 = host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t % 300))
     got = down(host, sched, host.CrossEntropy.backward(sched, state))
     assert got.dtype == x.dtype and (got[:, 300:] == 0).all()
+    # ... and so does the loss, as nll_loss_forward's does (cross_entropy.cpp:57-66)
+    loss16 = down(host, sched, loss16)
+    want16, _, _, _ = co.cross_entropy(x[:, :300], t % 300)
+    assert loss16.dtype == x.dtype
+    assert loss16 == want16.to(x.dtype) or abs(float(loss16) - float(want16)) <= 2.0 ** -7 * float(want16)
 
 
 # ---------------------------------------------------------------------- LayerNorm
