@@ -474,6 +474,25 @@ def per_op_table(args, torch, ops):
             del ms_, vs_
         del opt, w, grad, ws_, gs_
         torch.cuda.empty_cache()
+        # the same traffic without the arithmetic: four arrays of that many floats read, three
+        # rewritten.  What this reaches is the ceiling for the step's access pattern.
+        arrs = [torch.zeros(total, device=dev, dtype=torch.float32) for _ in range(4)]
+        nb4 = total * 4 // 16 * 16
+
+        def update4(i):
+            lib.cs_stream_update4(*[ctypes.c_void_p(a.data_ptr()) for a in arrs], nb4, stream)
+
+        update4(0)
+        med4, _ = event_ms(update4, max(5, reps // 4), torch)
+        out.append({"op": "stream_update4", "config": f"{tag} 4 x {total} floats read, 3 rewritten",
+                    "algorithmic_bytes": 7 * nb4, "ms_warm": round(med4, 5), "ms_cold": round(med4, 5),
+                    "gbps_warm": round(7 * nb4 / med4 / 1e6, 1), "gbps_cold": round(7 * nb4 / med4 / 1e6, 1),
+                    "frac_cold": round(7 * nb4 / med4 / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1})
+        rec["update4_ms_same_traffic"] = round(med4, 5)
+        rec["frac_of_update4"] = round(med4 / rec["ms_cold"], 3)
+        log(f"[per-op] stream_update4               {tag:34s} {med4*1e3:9.1f} us  {7 * nb4 / med4 / 1e6:8.1f} GB/s")
+        del arrs
+        torch.cuda.empty_cache()
 
     # ---- configuration 4: XL fused classifier [16384, 50257]
     if args.xl_ce and wanted("fused_classifier"):

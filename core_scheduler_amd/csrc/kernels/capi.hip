@@ -86,6 +86,46 @@ __global__ __launch_bounds__(kCopyThreads) void stream_fill_kernel(u32x4 *__rest
   }
 }
 
+// The traffic of an optimizer step without its arithmetic: four arrays read, three of them
+// written back in place (AdamW reads g, w, m, v and writes w, m, v).  Same chunking as the
+// AdamW kernel: two vectors per lane per array, every load issued before the first use.
+constexpr int kUpdateUnroll = 2;
+__global__ __launch_bounds__(kCopyThreads) void stream_update4_kernel(const u32x4 *__restrict__ a0,
+                                                                      u32x4 *__restrict__ a1,
+                                                                      u32x4 *__restrict__ a2,
+                                                                      u32x4 *__restrict__ a3, int64_t nvec) {
+  const int64_t base = (int64_t)blockIdx.x * (kCopyThreads * kUpdateUnroll) + threadIdx.x;
+  if (base - threadIdx.x + kCopyThreads * kUpdateUnroll <= nvec) {
+    u32x4 v0[kUpdateUnroll], v1[kUpdateUnroll], v2[kUpdateUnroll], v3[kUpdateUnroll];
+#pragma unroll
+    for (int u = 0; u < kUpdateUnroll; ++u) {
+      const int64_t i = base + (int64_t)u * kCopyThreads;
+      v0[u] = __builtin_nontemporal_load(a0 + i);
+      v1[u] = __builtin_nontemporal_load(a1 + i);
+      v2[u] = __builtin_nontemporal_load(a2 + i);
+      v3[u] = __builtin_nontemporal_load(a3 + i);
+    }
+#pragma unroll
+    for (int u = 0; u < kUpdateUnroll; ++u) {
+      const int64_t i = base + (int64_t)u * kCopyThreads;
+      const u32x4 x = v0[u] ^ v1[u] ^ v2[u] ^ v3[u];
+      __builtin_nontemporal_store(x + 1u, a1 + i);
+      __builtin_nontemporal_store(x + 2u, a2 + i);
+      __builtin_nontemporal_store(x + 3u, a3 + i);
+    }
+    return;
+  }
+  for (int u = 0; u < kUpdateUnroll; ++u) {
+    const int64_t i = base + (int64_t)u * kCopyThreads;
+    if (i < nvec) {
+      const u32x4 x = a0[i] ^ a1[i] ^ a2[i] ^ a3[i];
+      a1[i] = x + 1u;
+      a2[i] = x + 2u;
+      a3[i] = x + 3u;
+    }
+  }
+}
+
 // bytes from which the copy uses one vector per lane instead of two
 constexpr int64_t kCopyLargeBytes = 64ll << 20;
 
@@ -159,5 +199,19 @@ extern "C" int cs_stream_fill(void *dst, int64_t bytes, uint32_t value, void *st
   if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
   stream_fill_kernel<<<dim3((unsigned)blocks), dim3(kCopyThreads), 0, as_stream(stream)>>>(
       static_cast<u32x4 *>(dst), nvec, value);
+  return launch_status();
+}
+
+extern "C" int cs_stream_update4(const void *a0, void *a1, void *a2, void *a3, int64_t bytes, void *stream) {
+  if (bytes < 0 || bytes % 16 != 0) return CS_ERR_INVALID_ARGUMENT;
+  if (bytes == 0) return CS_OK;
+  if (!a0 || !a1 || !a2 || !a3) return CS_ERR_INVALID_ARGUMENT;
+  if (!is_aligned16(a0) || !is_aligned16(a1) || !is_aligned16(a2) || !is_aligned16(a3)) return CS_ERR_MISALIGNED;
+  const int64_t nvec = bytes / 16;
+  const int64_t blocks = ceil_div(nvec, (int64_t)kCopyThreads * kUpdateUnroll);
+  if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
+  stream_update4_kernel<<<dim3((unsigned)blocks), dim3(kCopyThreads), 0, as_stream(stream)>>>(
+      static_cast<const u32x4 *>(a0), static_cast<u32x4 *>(a1), static_cast<u32x4 *>(a2),
+      static_cast<u32x4 *>(a3), nvec);
   return launch_status();
 }

@@ -91,6 +91,14 @@ int64_t cs_stream_read_out_words(int64_t bytes);
 int cs_stream_read(const void *src, void *out, int64_t bytes, void *stream);
 int cs_stream_fill(void *dst, int64_t bytes, uint32_t value, void *stream);
 
+/* A fourth calibration with the memory traffic of the AdamW step and none of
+ * its arithmetic: a0..a3 (`bytes` each) are read, a1..a3 rewritten in place
+ * (a_k = (a0 ^ a1 ^ a2 ^ a3) + k per 32-bit word).  7 * bytes move; what this
+ * reaches is the ceiling for a kernel that streams four arrays in and three
+ * out.  No counterpart in the reference. */
+int cs_stream_update4(const void *a0, void *a1, void *a2, void *a3,
+                      int64_t bytes, void *stream);
+
 /* ------------------------------------------------------------------------
  * AdamW
  * replaces stepKernel / stepKernelAmsgrad and the step<UpT,T> kernels,

@@ -10,6 +10,7 @@ configurations; the largest ones are checked through the oracle on a sample of
 rows plus properties that hold at any size.
 """
 import math
+import numpy as np
 
 import pytest
 import torch
@@ -1168,3 +1169,14 @@ def test_stream_copy_read_fill(nbytes):
     torch.cuda.synchronize()
     assert int(dst[nbytes:].sum()) == 0
     assert bool((dst[:nbytes].view(torch.int32) == 0x01020304).all())
+    # four arrays in, three rewritten: a_k = (a0 ^ a1 ^ a2 ^ a3) + k per 32-bit word
+    arrs = [torch.randint(0, 256, (nbytes + 16,), dtype=torch.uint8, generator=g) for _ in range(4)]
+    gpu = [a.to(dev) for a in arrs]
+    _capi.check("cs_stream_update4", lib.cs_stream_update4(*[P(a.data_ptr()) for a in gpu], nbytes, st))
+    words = [a[:nbytes].numpy().view("<u4").astype("uint32") for a in arrs]
+    x = words[0] ^ words[1] ^ words[2] ^ words[3]
+    assert torch.equal(gpu[0].cpu(), arrs[0])
+    for k in (1, 2, 3):
+        got = gpu[k].cpu()
+        assert (got[:nbytes].numpy().view("<u4") == x + np.uint32(k)).all(), f"array {k}"
+        assert torch.equal(got[nbytes:], arrs[k][nbytes:]), "wrote past the end"
