@@ -689,7 +689,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "fused classifier (softmax + cross-entropy + in-place dlogits), logits [8192, 50257] bf16, "
-                        "row stride 50304, int64 targets, mean reduction (BASELINE configs[2])",
+                        "row stride 50304, int64 targets, mean reduction (benchmark configuration 2)",
             "algorithmic_bytes_per_step": CE_BYTES,
             "logits_buffers_rotated": head["buffers"],
             "loss": round(head["loss"], 5),
