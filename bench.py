@@ -165,6 +165,48 @@ def event_ms(fn, reps, torch, rounds=3):
     return statistics.median(batch), per_call
 
 
+class HipTimer:
+    """HIP events made with hipEventDisableSystemFence, the flag the runtime offers for events that
+    only measure time: recording one does not flush and invalidate the caches around the kernel it
+    brackets (a default event costs the stream ~2.7 us per record here, a fence-free one ~0.9 us)."""
+
+    _hip = None
+    FLAGS = 0x20000000  # hipEventDisableSystemFence; timing stays enabled
+
+    @classmethod
+    def hip(cls):
+        if cls._hip is None:
+            h = ctypes.CDLL("libamdhip64.so")
+            h.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+            h.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+            h.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+            h.hipEventDestroy.argtypes = [ctypes.c_void_p]
+            cls._hip = h
+        return cls._hip
+
+    def __init__(self):
+        self.ev = ctypes.c_void_p()
+        rc = self.hip().hipEventCreateWithFlags(ctypes.byref(self.ev), self.FLAGS)
+        if rc != 0:
+            raise RuntimeError(f"hipEventCreateWithFlags failed: {rc}")
+
+    def record(self, stream):
+        rc = self.hip().hipEventRecord(self.ev, stream)
+        if rc != 0:
+            raise RuntimeError(f"hipEventRecord failed: {rc}")
+
+    def ms_until(self, other):
+        out = ctypes.c_float()
+        rc = self.hip().hipEventElapsedTime(ctypes.byref(out), self.ev, other.ev)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return out.value
+
+    def __del__(self):
+        if self.ev:
+            self.hip().hipEventDestroy(self.ev)
+
+
 def run_headline(args, torch, ops, capi):
     dev = torch.device("cuda:0")
     lib = capi.load()
@@ -194,22 +236,22 @@ def run_headline(args, torch, ops, capi):
         buf = bufs[i % n_buf]
         phase(buf, 1)
         if ev:
-            ev[0].record()
+            ev[0].record(stream)
         phase(buf, 2)
         if ev:
-            ev[1].record()
+            ev[1].record(stream)
         phase(buf, 4)
 
     for i in range(W):
         step(i)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    evs = [(HipTimer(), HipTimer()) for _ in range(K)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(K):
         step(W + i, evs[i])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    kernel_ms = [a.elapsed_time(b) for a, b in evs]
+    kernel_ms = [a.ms_until(b) for a, b in evs]
     first_loss = loss.item()
     reused = K + W > n_buf
     return {
