@@ -76,9 +76,9 @@ Rows read_rows(const std::string &path) {
   CS_ASSERT_TRUE(infile.ok(), "Open File failed with error " + infile.status().ToString());
   auto reader = parquet::arrow::OpenFile(*infile, pool);
   CS_ASSERT_TRUE(reader.ok(), "Open File failed with error " + reader.status().ToString());
-  std::shared_ptr<arrow::Table> table;
-  const auto st = (*reader)->ReadTable(&table);
-  CS_ASSERT_TRUE(st.ok(), "Read File failed with error " + st.ToString());
+  const auto read = (*reader)->ReadTable();
+  CS_ASSERT_TRUE(read.ok(), "Read File failed with error " + read.status().ToString());
+  const std::shared_ptr<arrow::Table> &table = *read;
   CS_ASSERT_TRUE(table->num_columns() == 2 && table->schema()->field(0)->name() == "key" &&
                      table->schema()->field(1)->name() == "value",
                  path + " is not a parameter checkpoint (columns key, value)");

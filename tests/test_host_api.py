@@ -429,6 +429,65 @@ def test_adamw_module_matches_torch_optimizer(host, sched):
 
 
 @pytest.mark.gpu
+def test_training_chain_matches_torch_autograd(host, sched):
+    """Every op of the path in one chain, gradients flowing from the loss to the tables, five
+    optimizer steps: token + position gather -> LayerNorm -> GeLU (tanh) -> LayerNorm -> cross
+    entropy over the C columns, AdamW with weight decay.  The same model in torch (float64 on the
+    CPU, autograd, torch.optim.AdamW) from the same parameters has to show the same loss at every
+    step and end at the same parameters, which pins what the per-op tests cannot: that each
+    backward consumes exactly the gradient the next op produces and that the optimizer sees it."""
+    B, T, C, V = 4, 32, 128, 300
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    root, mods = build_tree(host, sched, V=V, T=T, C=C)
+    opt = host.AdamWModule(sched, root, **hp)
+    gelu = host.GeLU.init(sched, 1)
+    used = ["wte.weight", "wpe.weight", "h.0.ln_1.weight", "h.0.ln_1.bias", "ln_f.weight", "ln_f.bias"]
+    ref = {k: torch.nn.Parameter(down(host, sched, p).double()) for k, p in root.named_parameters() if k in used}
+    ref_opt = torch.optim.AdamW(ref.values(), lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"],
+                                weight_decay=hp["weight_decay"], foreach=False)
+    tok, pos = mods["wte"].state(), mods["wpe"].state()
+    losses, ref_losses = [], []
+
+    def reshaped(handle, *shape):  # a view of the same device memory under a new handle
+        return host.from_torch(sched, host.to_torch(sched, handle).view(*shape))
+
+    for step in range(5):
+        ids = randint(0, V, (B, T), 700)  # the same batch every step, so the loss has to fall
+        targets = randint(0, C, (B * T,), 720)
+        x = host.Embedding.forward_with_positions(sched, tok, pos, up(host, sched, ids))
+        h1 = mods["ln1"].forward(sched, x)
+        a = host.GeLU.forward(sched, gelu, h1)
+        h2 = mods["lnf"].forward(sched, a)
+        ce = host.CrossEntropy.init(sched)
+        loss = host.CrossEntropy.forward(sched, ce, reshaped(h2, B * T, C), up(host, sched, targets))
+        dlogits = host.CrossEntropy.backward(sched, ce)
+        da = mods["lnf"].backward(sched, reshaped(dlogits, B, T, C))
+        dh1 = host.GeLU.backward(sched, gelu, da)
+        dx = mods["ln1"].backward(sched, dh1)
+        host.Embedding.backward_with_positions(sched, tok, pos, dx)
+        opt.step(sched)
+        opt.zero_grad(sched)
+        losses.append(float(down(host, sched, loss)))
+        # the same step in torch
+        ref_opt.zero_grad()
+        rx = ref["wte.weight"][ids] + ref["wpe.weight"][None, :T]
+        r1 = torch.nn.functional.layer_norm(rx, (C,), ref["h.0.ln_1.weight"], ref["h.0.ln_1.bias"], 1e-5)
+        ra = torch.nn.functional.gelu(r1, approximate="tanh")
+        r2 = torch.nn.functional.layer_norm(ra, (C,), ref["ln_f.weight"], ref["ln_f.bias"], 1e-5)
+        rl = torch.nn.functional.cross_entropy(r2.reshape(B * T, C), targets)
+        rl.backward()
+        ref_opt.step()
+        ref_losses.append(float(rl.detach()))
+    for i, (a, b) in enumerate(zip(losses, ref_losses)):
+        assert abs(a - b) <= 2e-5 * abs(b), f"loss at step {i}: {a} vs {b}"
+    assert ref_losses[-1] < ref_losses[0]  # the model learns, so the gradients mattered
+    for k, p in root.named_parameters():
+        if k in used:
+            got = down(host, sched, p).double()
+            assert torch.allclose(got, ref[k].detach(), rtol=2e-4, atol=2e-5), f"{k}: {(got - ref[k]).abs().max()}"
+
+
+@pytest.mark.gpu
 def test_steps_without_host_waits_match_steps_with_waits(host, sched):
     """The scheduler's stream rules are what keeps a step correct when nothing waits on the host:
     gradients are produced on the assist stream (embedding backward) and on the main stream, the
