@@ -898,10 +898,10 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_positions_kernel(const T *__
   using U = typename Acc<T>::type;
   for (int64_t f = (int64_t)blockIdx.x * kThreads + threadIdx.x; f < TC;
        f += (int64_t)gridDim.x * kThreads) {
-    U a = 0;
-    for (int64_t b = 0; b < B; ++b) a += to_acc(dout[b * TC + f]);
-    if (accumulate) a += to_acc(dwpe[f]);
-    dwpe[f] = from_acc<T>(a);
+    double a = 0;  // sequential over the batch, so in double like the general row kernel
+    for (int64_t b = 0; b < B; ++b) a += (double)to_acc(dout[b * TC + f]);
+    if (accumulate) a += (double)to_acc(dwpe[f]);
+    dwpe[f] = from_acc<T>((U)a);
   }
 }
 
@@ -923,12 +923,14 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_rows_general_kernel(
     lo = go ? lo + half + 1 : lo;
     len = go ? len - half - 1 : half;
   }
+  // One thread adds a whole segment in order: thousands of sequential fp32 additions for a hot
+  // row drift by ~1e-4 of the terms' scale, so this path, which is not the fast one, adds in double.
   for (int64_t c = threadIdx.x; c < C; c += kThreads) {
-    U a = 0;
+    double a = 0;
     for (int64_t p = lo; p < n && sorted_id[p] == row; ++p)
-      a += to_acc(dout[(int64_t)sorted_pos[p] * C + c]);
-    if (accumulate) a += to_acc(dweight[(int64_t)row * C + c]);
-    dweight[(int64_t)row * C + c] = from_acc<T>(a);
+      a += (double)to_acc(dout[(int64_t)sorted_pos[p] * C + c]);
+    if (accumulate) a += (double)to_acc(dweight[(int64_t)row * C + c]);
+    dweight[(int64_t)row * C + c] = from_acc<T>((U)a);
   }
 }
 

@@ -78,6 +78,17 @@ def sum_tolerance(terms, dim=0):
     return 7.0 * 2.0 ** -24 * torch.sqrt(torch.log2(torch.tensor(float(n))) * (t * t).sum(dim))
 
 
+def scatter_sum_tolerance(terms, ids, num_rows):
+    """sum_tolerance for a scatter-add: out[ids[i]] += terms[i].  Row r of the result gets the bar
+    its own terms justify (rows nothing was added to get 0, plus the 1e-7 floor of the caller)."""
+    t = terms.reshape(ids.numel(), -1).double()
+    idx = ids.reshape(-1).long()
+    keep = (idx >= 0) & (idx < num_rows)
+    sq = torch.zeros((num_rows, t.shape[1]), dtype=torch.float64).index_add_(0, idx[keep], (t * t)[keep])
+    n = max(2, ids.numel())
+    return 7.0 * 2.0 ** -24 * torch.sqrt(torch.log2(torch.tensor(float(n))) * sq)
+
+
 def assert_sum_close(got, want, tol, name="", rtol=RTOL):
     """|got - want| <= tol + rtol |want| with a per-element `tol` (see sum_tolerance); 16-bit
     results may instead be within 1 ulp."""
