@@ -24,7 +24,7 @@ __global__ __launch_bounds__(kCopyThreads) void stream_copy_kernel(const u32x4 *
 #pragma unroll
     for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(src + base + (int64_t)u * kCopyThreads);
 #pragma unroll
-    for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], dst + base + (int64_t)u * kCopyThreads);
+    for (int u = 0; u < U; ++u) store_stream(dst + base + (int64_t)u * kCopyThreads, v[u]);
     return;
   }
   for (int u = 0; u < U; ++u) {
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kCopyThreads) void stream_fill_kernel(u32x4 *__rest
   const u32x4 v = {value, value, value, value};
   if (base - threadIdx.x + kCopyThreads * kFillUnroll <= nvec) {
 #pragma unroll
-    for (int u = 0; u < kFillUnroll; ++u) __builtin_nontemporal_store(v, dst + base + (int64_t)u * kCopyThreads);
+    for (int u = 0; u < kFillUnroll; ++u) store_stream(dst + base + (int64_t)u * kCopyThreads, v);
     return;
   }
   for (int u = 0; u < kFillUnroll; ++u) {
@@ -109,9 +109,9 @@ __global__ __launch_bounds__(kCopyThreads) void stream_update4_kernel(const u32x
     for (int u = 0; u < kUpdateUnroll; ++u) {
       const int64_t i = base + (int64_t)u * kCopyThreads;
       const u32x4 x = v0[u] ^ v1[u] ^ v2[u] ^ v3[u];
-      __builtin_nontemporal_store(x + 1u, a1 + i);
-      __builtin_nontemporal_store(x + 2u, a2 + i);
-      __builtin_nontemporal_store(x + 3u, a3 + i);
+      store_stream(a1 + i, x + 1u);
+      store_stream(a2 + i, x + 2u);
+      store_stream(a3 + i, x + 3u);
     }
     return;
   }

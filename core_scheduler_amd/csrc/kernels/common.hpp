@@ -107,9 +107,13 @@ __device__ __forceinline__ Vec16<T> load16_stream(const T *p) {
   const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
   return __builtin_bit_cast(Vec16<T>, raw);
 }
+// Every streaming store of the library goes through here.  Stores with the agent-scope
+// write-through bit (sc1, alone or with nt) were measured instead: a flat copy gains 2-6% at
+// 100-400 MB, but the kernels of this library ran up to 8% slower with them, so it stays nt.
+__device__ __forceinline__ void store_stream(u32x4 *p, const u32x4 v) { __builtin_nontemporal_store(v, p); }
 template <typename T>
 __device__ __forceinline__ void store16_stream(T *p, const Vec16<T> &v) {
-  __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4 *>(p));
+  store_stream(reinterpret_cast<u32x4 *>(p), __builtin_bit_cast(u32x4, v));
 }
 
 __host__ __device__ __forceinline__ bool is_aligned16(const void *p) {

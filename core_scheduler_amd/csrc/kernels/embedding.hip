@@ -340,7 +340,7 @@ __device__ __forceinline__ void zero_fill_block(u32x4 *__restrict__ dst, int64_t
 #pragma unroll 8
   for (int u = 0; u < kFillVecs / THREADS; ++u) {
     const int64_t i = v0 + (int64_t)u * THREADS + tid;
-    if (i < vecs) __builtin_nontemporal_store(z, dst + i);
+    if (i < vecs) store_stream(dst + i, z);
   }
 }
 
