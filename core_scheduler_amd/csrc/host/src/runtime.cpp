@@ -12,6 +12,8 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <ATen/ops/allclose.h>
 
+#include <atomic>
+#include <cstdint>
 #include <deque>
 #include <exception>
 #include <mutex>
@@ -30,7 +32,14 @@ namespace cs {
 // ------------------------------------------------------------------ events
 struct Event::Impl {
   void block() { event.block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()); }
-  void record() { event.record(); }
+  void record() {
+    static std::atomic<uint64_t> counter{0};
+    order = ++counter;
+    event.record();
+  }
+  // position of the last record() among all records of the process; 0 = never recorded.
+  // Two events recorded on one stream complete in this order.
+  uint64_t order = 0;
   [[nodiscard]] bool query() const { return event.query(); }
   void synchronize() const { event.synchronize(); }
 
@@ -166,8 +175,23 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
   // src/threading/dynamic_scheduler.cpp:150-160): every output, and the caller's own
   // bookkeeping, share it, since each record is a packet the stream has to work through.
   static Event run(const Task &task, const Priority lane) {
+    // of the inputs that another lane produced, the one stamped last per lane is waited for:
+    // a stream finishes its events in the order it recorded them, so that wait covers the rest
+    // (each wait is a packet that stalls this stream for microseconds even when it is granted)
+    const Event *latest[Priority::kNumPriority] = {};
     for (const auto &t : task.impl()->input()) {
-      if (t.impl()->priority() != lane && !t.impl()->event().query()) t.impl()->event().block();
+      const Priority from = t.impl()->priority();
+      if (from == lane) continue;
+      const Event &e = t.impl()->event();
+      if (from >= Priority::kNumPriority) {
+        // handed in from outside, stamped on whatever stream the caller was on: its own wait
+        if (!e.query()) e.block();
+      } else if (latest[from] == nullptr || e.impl()->order > latest[from]->impl()->order) {
+        latest[from] = &e;
+      }
+    }
+    for (const Event *e : latest) {
+      if (e != nullptr && !e->query()) e->block();
     }
     {
       // the task's name as a range in marker traces (rocprofv3 --marker-trace)
