@@ -99,6 +99,9 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 }
 
 // forward launch shape (rows a wave normalises per step, next step's rows prefetched or not)
+#ifndef CS_LN_FWD_ROWS_VPL1
+#define CS_LN_FWD_ROWS_VPL1 4
+#endif
 #ifndef CS_LN_FWD_ROWS_VPL2
 #define CS_LN_FWD_ROWS_VPL2 4
 #endif
@@ -107,6 +110,9 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 #endif
 #ifndef CS_LN_FWD_PF
 #define CS_LN_FWD_PF true
+#endif
+#ifndef CS_LN_ADD_ROWS_VPL1
+#define CS_LN_ADD_ROWS_VPL1 4
 #endif
 #ifndef CS_LN_ADD_ROWS_VPL2
 #define CS_LN_ADD_ROWS_VPL2 4
@@ -769,14 +775,17 @@ struct FastPlan {
 constexpr int kMaxVplWithResidual = 4;
 
 // x vectors per lane needed for C columns of x_dtype; the fast kernels are
-// instantiated for 2, 4 and 8.
+// instantiated for 1, 2, 4 and 8.
 FastPlan fast_plan(int64_t C, int x_dtype) {
   FastPlan p;
   const int vn = 16 / (int)dtype_size(x_dtype);
   if (x_dtype == CS_F64 || C <= 0 || C % vn != 0) return p;
   const int64_t nvec = C / vn;
   const int64_t per_lane = ceil_div(nvec, (int64_t)kWave);
-  if (per_lane <= 2) {
+  if (per_lane <= 1) {
+    p.vpl = 1;
+    p.fwd_rows = CS_LN_FWD_ROWS_VPL1;
+  } else if (per_lane <= 2) {
     p.vpl = 2;
     p.fwd_rows = CS_LN_FWD_ROWS_VPL2;
   } else if (per_lane <= 4) {
@@ -813,20 +822,28 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
       // with the residual stream a wave holds two inputs per row: half the rows per step
-      const int r_rows = res ? (p.vpl == 2 ? CS_LN_ADD_ROWS_VPL2 : p.vpl == 4 ? CS_LN_ADD_ROWS_VPL4 : 1) : p.fwd_rows;
+      const int r_rows = res ? (p.vpl == 1   ? CS_LN_ADD_ROWS_VPL1
+                                : p.vpl == 2 ? CS_LN_ADD_ROWS_VPL2
+                                : p.vpl == 4 ? CS_LN_ADD_ROWS_VPL4
+                                             : 1)
+                             : p.fwd_rows;
       const dim3 grid((unsigned)ln_blocks(rows, r_rows, kLnFwdMaxBlocks)), block(kLnThreads);
 #define CS_LN_FWD(VPL, R, HAS_RES)                                                          \
   ln_fwd_rows_kernel<TX, TY, TP, VPL, R, CS_LN_FWD_PF, HAS_RES><<<grid, block, 0, s>>>(     \
       (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean,           \
       (float *)rstd, rows, (int)C, (float)eps, (const TX *)res, (TX *)sum_out)
       if (res) {
-        if (p.vpl == 2) {
+        if (p.vpl == 1) {
+          CS_LN_FWD(1, CS_LN_ADD_ROWS_VPL1, true);
+        } else if (p.vpl == 2) {
           CS_LN_FWD(2, CS_LN_ADD_ROWS_VPL2, true);
         } else if (p.vpl == 4) {
           CS_LN_FWD(4, CS_LN_ADD_ROWS_VPL4, true);
         } else {
           CS_LN_FWD(8, 1, true);
         }
+      } else if (p.vpl == 1) {
+        CS_LN_FWD(1, CS_LN_FWD_ROWS_VPL1, false);
       } else if (p.vpl == 2) {
         CS_LN_FWD(2, CS_LN_FWD_ROWS_VPL2, false);
       } else if (p.vpl == 4) {
@@ -856,7 +873,7 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
 int bwd_partial_rows(int64_t rows, int vpl) {
   // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
   if (vpl == 8) return ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
-  return ln_blocks(rows, 1, vpl == 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
+  return ln_blocks(rows, 1, vpl <= 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
 }
 
 enum BwdPhase { kBwdWhole = 0, kBwdRowsOnly = 1 };
@@ -880,7 +897,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
       const int blocks =
-          ln_blocks(rows, 1, p.vpl == 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
+          ln_blocks(rows, 1, p.vpl <= 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
       const int split_blocks = bwd_partial_rows(rows, 8);
       const int blocks_used = want_dp ? bwd_partial_rows(rows, p.vpl) : blocks;  // partial rows left behind
       const size_t need = want_dp ? (size_t)blocks_used * 2 * C * sizeof(float) : 0;
@@ -900,7 +917,13 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   } else {                                      \
     CS_LN_BWD(VPL, WPE, false, true, false);    \
   }
-      if (p.vpl == 2 && dres && want_dp) {
+      if (p.vpl == 1 && dres && want_dp) {
+        CS_LN_BWD(1, 4, true, true, true);
+      } else if (p.vpl == 1 && dres) {
+        CS_LN_BWD(1, 4, true, false, true);
+      } else if (p.vpl == 1) {
+        CS_LN_BWD_MASK(1, 4)
+      } else if (p.vpl == 2 && dres && want_dp) {
         CS_LN_BWD(2, 3, true, true, true);  // four per SIMD would spill
       } else if (p.vpl == 2 && dres) {
         CS_LN_BWD(2, 4, true, false, true);

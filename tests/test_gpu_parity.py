@@ -328,6 +328,10 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
     (3, 4096, torch.float16, torch.float16),        # fewer rows than wave pairs
     (1100, 2056, torch.bfloat16, torch.float32),    # just over 4 vectors per lane, several rows per pair
     (5, 768, torch.float32, torch.float32),         # fewer rows than one workgroup
+    (4096, 384, torch.bfloat16, torch.float32),     # one vector per lane, 48 of 64 lanes busy
+    (1000, 512, torch.float16, torch.float16),      # one vector per lane, every lane busy
+    (777, 256, torch.float32, torch.float32),       # the same plan from fp32 rows
+    (300, 8, torch.bfloat16, torch.bfloat16),       # a single vector per row
     (64, 50, torch.float32, torch.float32),         # C not a multiple of the vector width
     (2049, 50, torch.float32, torch.float32),       # the same with long column sums
     (33, 10000, torch.bfloat16, torch.float32),     # beyond the register plans
@@ -344,6 +348,8 @@ def test_layernorm(ops, co, rows, C, x_dtype, p_dtype):
     (513, 768, torch.float16, torch.float16),
     (77, 4096, torch.bfloat16, torch.float32),      # 8 vectors per lane plan
     (5, 768, torch.float32, torch.float32),
+    (2000, 384, torch.bfloat16, torch.float32),     # one vector per lane
+    (100, 64, torch.float16, torch.float16),
     (64, 50, torch.float32, torch.float32),         # general path
     (33, 10000, torch.bfloat16, torch.float32),     # general path
     (128, 384, torch.float64, torch.float64),
@@ -478,6 +484,7 @@ def test_layernorm_masks_and_accumulate(ops, co):
     (77, 4096, torch.bfloat16, torch.float32, False),     # two waves per row
     (2051, 1600, torch.float32, torch.float32, False),
     (3, 768, torch.float32, torch.float32, False),
+    (1500, 384, torch.bfloat16, torch.float32, True),     # one vector per lane
 ])
 def test_layernorm_backward_as_two_calls(ops, rows, C, x_dtype, p_dtype, wide_dy):
     """Row pass on one stream, sum of the partial rows on another (the reference's main and
