@@ -64,18 +64,35 @@ __device__ __forceinline__ void adam_update(T &w, T &m, T &v, T &vmax, const T g
 }
 
 constexpr int kAdamThreads = 256;
-// 16-byte vectors per lane per chunk.  Measured on MI355X at 124M fp32 parameters: 2 -> 5.97 TB/s,
-// 1 -> 5.36, 3 -> 5.72, 4 -> 5.59, 8 -> 5.61 (256 lanes; 128 x 2 and 512 x 2 are within 3%).
-constexpr int kAdamUnroll = 2;
+// A chunk is what one workgroup updates: kAdamThreads lanes x U 16-byte vectors per array.
+// One launch per tensor (cs_adamw_step, the reference's shape): U = 2 with a lane's accesses a
+// workgroup apart; of 1, 2, 3, 4, 8 it measured best there (5.97 TB/s at 124M fp32 parameters
+// against 5.36 - 5.72), and the many small launches of a model want small chunks.
+// One launch for all tensors: U = 4 with every wave owning 4 consecutive kilobytes of each
+// array.  The traffic alone (four arrays read, three rewritten) runs 568 us in that shape
+// against 612 us in the other at 124M floats per array; the step gains 3% (620 -> 602 us,
+// 7.96 -> 7.74 ms for 1.56G parameters).
+constexpr int kAdamFlatUnroll = 2;
+constexpr int kAdamMultiUnroll = 4;
 
-template <typename T>
+// Vector index inside a chunk for a lane's u-th access.
+template <int U, bool WAVE_CONTIG>
+__device__ __forceinline__ int adam_vec_index(int u, int tid) {
+  if constexpr (WAVE_CONTIG) {
+    return (tid >> 6) * (kWave * U) + u * kWave + (tid & (kWave - 1));
+  } else {
+    return u * kAdamThreads + tid;
+  }
+}
+
+template <typename T, int U>
 constexpr int64_t adam_chunk_elems() {
-  return (int64_t)kAdamThreads * kAdamUnroll * Vec16<T>::n;
+  return (int64_t)kAdamThreads * U * Vec16<T>::n;
 }
 
 // Updates elements [begin, end) of one tensor with this workgroup.  `vec_ok`
 // says all five pointers are 16-byte aligned at element 0.
-template <typename T, bool AMSGRAD>
+template <typename T, bool AMSGRAD, int U_, bool WAVE_CONTIG>
 __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restrict__ dw,
                                            T *__restrict__ m, T *__restrict__ v,
                                            T *__restrict__ vmax, int64_t begin, int64_t end,
@@ -84,12 +101,12 @@ __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restric
                                            const typename Acc<T>::type gscale) {
   constexpr int VN = Vec16<T>::n;
   const int tid = threadIdx.x;
-  if (vec_ok && end - begin == adam_chunk_elems<T>()) {
+  if (vec_ok && end - begin == adam_chunk_elems<T, U_>()) {
     // full chunk: issue every load before the first use
-    Vec16<T> vw[kAdamUnroll], vg[kAdamUnroll], vm[kAdamUnroll], vv[kAdamUnroll], vx[kAdamUnroll];
+    Vec16<T> vw[U_], vg[U_], vm[U_], vv[U_], vx[U_];
 #pragma unroll
-    for (int u = 0; u < kAdamUnroll; ++u) {
-      const int64_t off = begin + ((int64_t)u * kAdamThreads + tid) * VN;
+    for (int u = 0; u < U_; ++u) {
+      const int64_t off = begin + (int64_t)adam_vec_index<U_, WAVE_CONTIG>(u, tid) * VN;
       vg[u] = load16_stream(dw + off);
       vw[u] = load16_stream(w + off);
       vm[u] = load16_stream(m + off);
@@ -97,8 +114,8 @@ __device__ __forceinline__ void adam_chunk(T *__restrict__ w, const T *__restric
       if constexpr (AMSGRAD) vx[u] = load16_stream(vmax + off);
     }
 #pragma unroll
-    for (int u = 0; u < kAdamUnroll; ++u) {
-      const int64_t off = begin + ((int64_t)u * kAdamThreads + tid) * VN;
+    for (int u = 0; u < U_; ++u) {
+      const int64_t off = begin + (int64_t)adam_vec_index<U_, WAVE_CONTIG>(u, tid) * VN;
 #pragma unroll
       for (int k = 0; k < VN; ++k) {
         adam_update<T, AMSGRAD>(vw[u].e[k], vm[u].e[k], vv[u].e[k], vx[u].e[k], vg[u].e[k], h, gscale);
@@ -126,10 +143,11 @@ template <typename T, bool AMSGRAD>
 __global__ __launch_bounds__(kAdamThreads) void adamw_flat_kernel(
     T *__restrict__ w, const T *__restrict__ dw, T *__restrict__ m, T *__restrict__ v,
     T *__restrict__ vmax, int64_t n, bool vec_ok, AdamHyper<typename Acc<T>::type> h) {
-  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t chunk = adam_chunk_elems<T, kAdamFlatUnroll>();
   const int64_t begin = (int64_t)blockIdx.x * chunk;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
-  adam_chunk<T, AMSGRAD>(w, dw, m, v, vmax, begin, end, vec_ok, h, (typename Acc<T>::type)1);
+  adam_chunk<T, AMSGRAD, kAdamFlatUnroll, false>(w, dw, m, v, vmax, begin, end, vec_ok, h,
+                                                 (typename Acc<T>::type)1);
 }
 
 // ---------------------------------------------------------- multi-tensor
@@ -180,14 +198,14 @@ __global__ __launch_bounds__(kAdamThreads) void adamw_multi_kernel(
   const int lo = tensor_of_slot(table, n_tensors, slot);
   const DevTensor *desc =
       reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
-  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t chunk = adam_chunk_elems<T, kAdamMultiUnroll>();
   const int64_t begin = (slot - table[lo]) * chunk;
   const int64_t n = desc->n;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
   const U gscale = clip ? (U)*clip : (U)1;
-  adam_chunk<T, AMSGRAD>(static_cast<T *>(desc->w), static_cast<const T *>(desc->dw),
-                         static_cast<T *>(desc->m), static_cast<T *>(desc->v),
-                         static_cast<T *>(desc->vmax), begin, end, desc->vec_ok != 0, h, gscale);
+  adam_chunk<T, AMSGRAD, kAdamMultiUnroll, true>(
+      static_cast<T *>(desc->w), static_cast<const T *>(desc->dw), static_cast<T *>(desc->m),
+      static_cast<T *>(desc->v), static_cast<T *>(desc->vmax), begin, end, desc->vec_ok != 0, h, gscale);
 }
 
 // ------------------------------------------------- global gradient norm
@@ -206,7 +224,7 @@ __global__ __launch_bounds__(kAdamThreads) void grad_norm_partial_kernel(
   const DevTensor *desc =
       reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
   const T *g = static_cast<const T *>(desc->dw);
-  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t chunk = adam_chunk_elems<T, kAdamMultiUnroll>();
   const int64_t begin = (slot - table[lo]) * chunk;
   const int64_t n = desc->n;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
@@ -221,12 +239,12 @@ __global__ __launch_bounds__(kAdamThreads) void grad_norm_partial_kernel(
     }
   };
   if (is_aligned16(g) && end - begin == chunk) {
-    Vec16<T> v[kAdamUnroll];
+    Vec16<T> v[kAdamMultiUnroll];
 #pragma unroll
-    for (int u = 0; u < kAdamUnroll; ++u)
-      v[u] = load16(g + begin + ((int64_t)u * kAdamThreads + tid) * VN);  // read again by the step: keep it cached
+    for (int u = 0; u < kAdamMultiUnroll; ++u)
+      v[u] = load16(g + begin + (int64_t)adam_vec_index<kAdamMultiUnroll, true>(u, tid) * VN);  // read again by the step: keep it cached
 #pragma unroll
-    for (int u = 0; u < kAdamUnroll; ++u)
+    for (int u = 0; u < kAdamMultiUnroll; ++u)
 #pragma unroll
       for (int k = 0; k < VN; ++k) take(v[u].e[k]);
   } else {
@@ -307,7 +325,7 @@ __global__ __launch_bounds__(kAdamThreads) void grad_scale_kernel(const int64_t 
   const DevTensor *desc =
       reinterpret_cast<const DevTensor *>(table + slot_array_len(n_tensors)) + lo;
   T *g = static_cast<T *>(const_cast<void *>(desc->dw));
-  const int64_t chunk = adam_chunk_elems<T>();
+  const int64_t chunk = adam_chunk_elems<T, kAdamMultiUnroll>();
   const int64_t begin = (slot - table[lo]) * chunk;
   const int64_t n = desc->n;
   const int64_t end = begin + chunk < n ? begin + chunk : n;
@@ -315,8 +333,8 @@ __global__ __launch_bounds__(kAdamThreads) void grad_scale_kernel(const int64_t 
   const U scale = (U)*clip;
   if (is_aligned16(g) && end - begin == chunk) {
 #pragma unroll
-    for (int u = 0; u < kAdamUnroll; ++u) {
-      T *p = g + begin + ((int64_t)u * kAdamThreads + tid) * VN;
+    for (int u = 0; u < kAdamMultiUnroll; ++u) {
+      T *p = g + begin + (int64_t)adam_vec_index<kAdamMultiUnroll, true>(u, tid) * VN;
       Vec16<T> v = load16(p);
 #pragma unroll
       for (int k = 0; k < VN; ++k) v.e[k] = from_acc<T>(to_acc(v.e[k]) * scale);
@@ -341,9 +359,10 @@ AdamHyper<U> make_hyper(double lr, double beta1, double beta2, double eps, doubl
   return h;
 }
 
+// workgroup slots a tensor of n elements takes in the multi-tensor table
 template <typename T>
 int64_t chunks_for(int64_t n) {
-  return ceil_div(n, adam_chunk_elems<T>());
+  return ceil_div(n, adam_chunk_elems<T, kAdamMultiUnroll>());
 }
 
 int64_t chunks_for_dtype(int dtype, int64_t n) {
@@ -360,7 +379,7 @@ template <typename T>
 int launch_flat(void *w, const void *dw, void *m, void *v, void *vmax, int64_t n, double lr,
                 double beta1, double beta2, double eps, double wd, int64_t t, hipStream_t s) {
   using U = typename Acc<T>::type;
-  const int64_t blocks = chunks_for<T>(n);
+  const int64_t blocks = ceil_div(n, adam_chunk_elems<T, kAdamFlatUnroll>());
   if (blocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
   const bool vec_ok = is_aligned16(w) && is_aligned16(dw) && is_aligned16(m) && is_aligned16(v) &&
                       (vmax == nullptr || is_aligned16(vmax));

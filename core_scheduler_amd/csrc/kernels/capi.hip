@@ -88,18 +88,23 @@ __global__ __launch_bounds__(kCopyThreads) void stream_fill_kernel(u32x4 *__rest
 
 // The traffic of an optimizer step without its arithmetic: four arrays read, three of them
 // written back in place (AdamW reads g, w, m, v and writes w, m, v).  Same chunking as the
-// AdamW kernel: two vectors per lane per array, every load issued before the first use.
-constexpr int kUpdateUnroll = 2;
+// multi-tensor AdamW kernel: four vectors per lane per array, every wave owning four consecutive
+// kilobytes of each array, every load issued before the first use.
+constexpr int kUpdateUnroll = 4;
+__device__ __forceinline__ int64_t update_index(int64_t chunk_base, int u, int tid) {
+  return chunk_base + (tid >> 6) * (kWave * kUpdateUnroll) + u * kWave + (tid & (kWave - 1));
+}
 __global__ __launch_bounds__(kCopyThreads) void stream_update4_kernel(const u32x4 *__restrict__ a0,
                                                                       u32x4 *__restrict__ a1,
                                                                       u32x4 *__restrict__ a2,
                                                                       u32x4 *__restrict__ a3, int64_t nvec) {
-  const int64_t base = (int64_t)blockIdx.x * (kCopyThreads * kUpdateUnroll) + threadIdx.x;
-  if (base - threadIdx.x + kCopyThreads * kUpdateUnroll <= nvec) {
+  const int64_t chunk_base = (int64_t)blockIdx.x * (kCopyThreads * kUpdateUnroll);
+  const int tid = threadIdx.x;
+  if (chunk_base + kCopyThreads * kUpdateUnroll <= nvec) {
     u32x4 v0[kUpdateUnroll], v1[kUpdateUnroll], v2[kUpdateUnroll], v3[kUpdateUnroll];
 #pragma unroll
     for (int u = 0; u < kUpdateUnroll; ++u) {
-      const int64_t i = base + (int64_t)u * kCopyThreads;
+      const int64_t i = update_index(chunk_base, u, tid);
       v0[u] = __builtin_nontemporal_load(a0 + i);
       v1[u] = __builtin_nontemporal_load(a1 + i);
       v2[u] = __builtin_nontemporal_load(a2 + i);
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(kCopyThreads) void stream_update4_kernel(const u32x
     }
 #pragma unroll
     for (int u = 0; u < kUpdateUnroll; ++u) {
-      const int64_t i = base + (int64_t)u * kCopyThreads;
+      const int64_t i = update_index(chunk_base, u, tid);
       const u32x4 x = v0[u] ^ v1[u] ^ v2[u] ^ v3[u];
       store_stream(a1 + i, x + 1u);
       store_stream(a2 + i, x + 2u);
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(kCopyThreads) void stream_update4_kernel(const u32x
     return;
   }
   for (int u = 0; u < kUpdateUnroll; ++u) {
-    const int64_t i = base + (int64_t)u * kCopyThreads;
+    const int64_t i = chunk_base + (int64_t)u * kCopyThreads + tid;
     if (i < nvec) {
       const u32x4 x = a0[i] ^ a1[i] ^ a2[i] ^ a3[i];
       a1[i] = x + 1u;

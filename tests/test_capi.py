@@ -93,7 +93,7 @@ def test_multi_tensor_table_layout():
     lib = _capi.load()
     n = 3
     arr = (_capi.AdamWTensor * n)()
-    sizes = [2048 * 4 + 1, 5, 4096]
+    sizes = [4096 * 4 + 1, 5, 8192]
     for i, s in enumerate(sizes):
         base = 0x10000 * (i + 1)
         arr[i].w, arr[i].dw, arr[i].m, arr[i].v, arr[i].v_max, arr[i].n = base, base + 0x1000, base + 0x2000, base + 0x3000, None, s
@@ -101,7 +101,7 @@ def test_multi_tensor_table_layout():
     buf = (ctypes.c_uint8 * nbytes)()
     slots = ctypes.c_int64()
     assert lib.cs_adamw_multi_build_table(arr, n, _capi.F32, buf, nbytes, ctypes.byref(slots)) == 0
-    assert slots.value == 5 + 1 + 2  # 2048-element chunks
+    assert slots.value == 5 + 1 + 2  # one workgroup slot per 4096 fp32 elements (256 lanes x 4 vectors)
     first = (ctypes.c_int64 * 8).from_buffer(buf)
     assert list(first[:4]) == [0, 5, 6, 8]
     assert lib.cs_adamw_multi_build_table(arr, n, _capi.F32, buf, nbytes - 1, ctypes.byref(slots)) == _capi.ERR_WORKSPACE
