@@ -579,6 +579,81 @@ def per_op_table(args, torch, ops):
                         "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 3})
             log(f"[per-op] fused_classifier call        {tag:42s} {med*1e3:9.1f} us  {nbytes/med/1e6:8.1f} GB/s")
         del grads
+
+    # ---- every launch of the path in one GPT-2-small training step (B 8, T 1024, C 768, 12
+    #      blocks, vocabulary 50257), back to back on one stream, each on buffers of its own as a
+    #      training step holds them: gather-add, 25 LayerNorm forward (24 of them with the residual
+    #      add), 12 GeLU forward, the fused classifier, then the backward launches of the same and
+    #      one AdamW step over all 148 parameter tensors.  The matrix products and attention that
+    #      sit between them in a model are not part of the path and are not run.
+    if wanted("gpt2_small_step_path"):
+        torch.cuda.empty_cache()
+        B, T, C, L, V = 8, 1024, 768, 12, CE_V
+        rows = B * T
+        wte, wpe = randn((V, C), 0.02), randn((T, C), 0.02)
+        ids = torch.randint(0, V, (B, T), generator=g, device=dev, dtype=torch.int64)
+        gamma, beta = randn(C, 0.02, 1.0, torch.float32), randn(C, 0.02, 0.0, torch.float32)
+        n_ln = 2 * L + 1
+        xs = [randn((rows, C)) for _ in range(n_ln)]        # LayerNorm inputs (the residual stream)
+        res = [randn((rows, C)) for _ in range(n_ln)]       # what is added to it before each norm
+        dys = [randn((rows, C)) for _ in range(n_ln)]
+        hs = [randn((rows, 4 * C), 1.5) for _ in range(L)]  # GeLU inputs
+        dhs = [randn((rows, 4 * C)) for _ in range(L)]
+        logits = randn((rows, CE_STRIDE), 2.0)
+        targets = torch.randint(0, V, (rows,), generator=g, device=dev, dtype=torch.int64)
+        dout = randn((B, T, C))
+        _, mean, rstd = ops.layernorm_forward(xs[0], gamma, beta, 1e-5)
+        sizes = gpt2_param_sizes(L, C)
+        total = sum(sizes)
+        w = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 0.02, generator=g)
+        grad = torch.empty(total, device=dev, dtype=torch.float32).normal_(0, 1e-3, generator=g)
+        offs = [0]
+        for sz in sizes:
+            offs.append(offs[-1] + sz)
+        opt = ops.MultiTensorAdamW([w[offs[i]:offs[i + 1]] for i in range(len(sizes))],
+                                   [grad[offs[i]:offs[i + 1]] for i in range(len(sizes))],
+                                   lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+        keep = {}
+
+        def path_step(i):
+            k = []
+            k.append(ops.embedding_forward_add(wte, wpe, ids))
+            k.append(ops.layernorm_forward(xs[0], gamma, beta, 1e-5))
+            for j in range(1, n_ln):
+                k.append(ops.add_layernorm_forward(xs[j], res[j], gamma, beta, 1e-5))
+            for j in range(L):
+                k.append(ops.gelu_forward(hs[j], "tanh"))
+            k.append(ops.fused_classifier(logits, targets, V, inplace=True))
+            for j in range(L):
+                k.append(ops.gelu_backward(dhs[j], hs[j], "tanh"))
+            for j in range(1, n_ln):
+                k.append(ops.layernorm_backward(dys[j], xs[j], mean, rstd, gamma, dresidual=res[j]))
+            k.append(ops.layernorm_backward(dys[0], xs[0], mean, rstd, gamma))
+            k.append(ops.embedding_backward_fused(dout, ids, V))
+            opt.step()
+            keep[i % 2] = k  # outputs stay alive for a step, as activations and gradients do
+
+        ln_f = 2 * rows * C * 2 + 2 * C * 4 + 2 * rows * 4
+        ln_b = 3 * rows * C * 2 + 2 * rows * 4 + 3 * C * 4
+        nbytes = ((rows * C * 2 + rows * 8 + T * C * 2 + rows * C * 2)                # gather-add
+                  + ln_f + (n_ln - 1) * (ln_f + 2 * rows * C * 2)                     # LayerNorm forward
+                  + L * 2 * rows * 4 * C * 2 + L * 3 * rows * 4 * C * 2               # GeLU forward, backward
+                  + 2 * rows * CE_V * 2 + rows * 12                                   # fused classifier
+                  + ln_b + (n_ln - 1) * (ln_b + rows * C * 2)                         # LayerNorm backward
+                  + rows * C * 2 + V * C * 2 + T * C * 2                              # embedding backward
+                  + 28 * total)                                                       # AdamW
+        launches = 1 + n_ln + L + 3 + L + 2 * n_ln + 3 + 1
+        path_step(0)
+        med, _ = event_ms(path_step, 5, torch)
+        out.append({"op": "gpt2_small_step_path", "config": f"B{B} T{T} C{C} {L} blocks V{V}: {launches} launches of the path, "
+                                                           "one training step, no matrix products",
+                    "algorithmic_bytes": nbytes, "ms_warm": round(med, 5), "ms_cold": round(med, 5),
+                    "gbps_warm": round(nbytes / med / 1e6, 1), "gbps_cold": round(nbytes / med / 1e6, 1),
+                    "frac_cold": round(nbytes / med / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1, "launches": launches})
+        log(f"[per-op] gpt2_small_step_path         {launches} launches {med*1e3:9.1f} us  {nbytes/med/1e6:8.1f} GB/s  "
+            f"{nbytes/med/1e6/HBM_PEAK_GBPS*100:5.1f}% of HBM peak")
+        del opt, w, grad, xs, res, dys, hs, dhs, logits, keep
+        torch.cuda.empty_cache()
     return out
 
 
