@@ -166,6 +166,36 @@ __device__ __forceinline__ void load_rows(RowSet<T, VN, VPL, R> &dst, const T *_
   }
 }
 
+// One row, every lane loading: lanes past the end of the row read its last vector again.  A load
+// under a lane-dependent condition can make the compiler wait for it before it issues the next
+// one (it did for the third input of the backward kernel: two extra round trips per row), an
+// unconditional one cannot.  What the extra lanes hold is masked where it matters (zero_past_row).
+template <typename T, int VN, int VPL>
+__device__ __forceinline__ void load_row_all_lanes(RowSet<T, VN, VPL, 1> &dst, const T *__restrict__ src,
+                                                   int64_t row, int C, int nvec, int lane) {
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int idx = lane + kWave * j;
+    dst.v[0][j] = load_raw<T, VN>(src + row * C + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
+  }
+}
+template <typename T, int VN, int VPL>
+__device__ __forceinline__ void zero_past_row(RowSet<T, VN, VPL, 1> &r, int nvec, int lane) {
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const bool past = lane + kWave * j >= nvec;
+#pragma unroll
+    for (int q = 0; q < VN / Vec16<T>::n; ++q) {
+      u32x4 w = __builtin_bit_cast(u32x4, r.v[0][j].v[q]);
+      w.x = past ? 0u : w.x;
+      w.y = past ? 0u : w.y;
+      w.z = past ? 0u : w.z;
+      w.w = past ? 0u : w.w;
+      r.v[0][j].v[q] = __builtin_bit_cast(Vec16<T>, w);
+    }
+  }
+}
+
 // HAS_RES: the rows that are normalised are x + residual, rounded to x's type (the sum is also
 // written to sum_out, which may be x or residual itself): the residual add in front of the
 // LayerNorm of a transformer block without a [rows, C] round trip between two launches.
@@ -330,9 +360,20 @@ __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
     RowSet<TDY, VN, VPL, 1> dcur;
     RowSet<TX, VN, VPL, 1> xcur;
     RowSet<TDX, VN, VPL, 1> rcur;  // this row of dresidual, in flight during the reductions
-    load_rows<TDY, VN, VPL, 1>(dcur, dy, row, rows, C, nvec, lane);
-    load_rows<TX, VN, VPL, 1>(xcur, x, row, rows, C, nvec, lane);
-    if constexpr (HAS_DRES) load_rows<TDX, VN, VPL, 1>(rcur, dres, row, rows, C, nvec, lane);
+    if constexpr (HAS_DRES) {
+      // three inputs: with loads under the lane's own condition the compiler waits for each
+      // piece of the third before it issues the next (two extra round trips per row at
+      // [8192,768]: 21.0 -> 19.7 us, 53.1 -> 46.4 us at [16384,1600]); every lane loads instead
+      load_row_all_lanes<TDY, VN, VPL>(dcur, dy, row, C, nvec, lane);
+      load_row_all_lanes<TX, VN, VPL>(xcur, x, row, C, nvec, lane);
+      load_row_all_lanes<TDX, VN, VPL>(rcur, dres, row, C, nvec, lane);
+      zero_past_row<TDY, VN, VPL>(dcur, nvec, lane);  // so that lanes past the row add nothing below
+    } else {
+      // two inputs: the conditional form has no such waits and needs half the registers
+      // (13.9 against 14.8 us, 34.0 against 36.4 us)
+      load_rows<TDY, VN, VPL, 1>(dcur, dy, row, rows, C, nvec, lane);
+      load_rows<TX, VN, VPL, 1>(xcur, x, row, rows, C, nvec, lane);
+    }
     const float mu = mean[row], rs = rstd[row];
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -362,6 +403,9 @@ __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
       for (int j = 0; j < VPL; ++j) {
         forget_unpacked(xcur.v[0][j]);
         forget_unpacked(dcur.v[0][j]);
+        // also keeps the load of this piece up where it was issued: without a use outside the
+        // branch below the compiler moves it into the branch, behind the reductions
+        if constexpr (HAS_DRES) forget_unpacked(rcur.v[0][j]);
         const int idx = lane + kWave * j;
         if (idx < nvec) {
           float o[VN];
