@@ -155,7 +155,9 @@ __global__ __launch_bounds__(BLOCK) void ce_rows_kernel(
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int idx = tid + BLOCK * j;
-    if (idx < nvec) xr[j] = load16_stream(x + (int64_t)idx * VN);
+    // every lane loads (lanes past the row read its last vector, which nothing below uses): a
+    // load under the lane's own condition makes the compiler wait for it before the next one
+    xr[j] = load16_stream(x + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
   }
   const float x_t = tid == 0 ? to_acc(x[target]) : 0.f;
 
@@ -341,6 +343,8 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
           const int idx = tid + BLOCK * j;
+          // (kept under the lane's condition here: the compiler issues these back to back as they
+          // are, and the unconditional form spills 56 bytes per lane: 283 -> 305 us)
           if (idx < nvec) nxt[j] = load_e_stream<T, EPV>(x + (int64_t)idx * VN);
         }
         if (tid == 0) nx_t = to_acc(x[ntgt]);
@@ -513,7 +517,8 @@ __global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
 #pragma unroll
       for (int u = 0; u < kWideU; ++u) {
         const int idx = base + BLOCK * u;
-        if (idx < nvec) v[u] = load16(xb + (int64_t)idx * VN);  // cached: read again below
+        // cached: read again below.  Every lane loads, see ce_rows_kernel.
+        v[u] = load16(xb + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
       }
       float xs[kWideU][VN];
       float cm = -INFINITY;
@@ -585,7 +590,7 @@ __global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
 #pragma unroll
       for (int u = 0; u < kWideU; ++u) {
         const int idx = base + BLOCK * u;
-        if (idx < nvec) v[u] = load16_stream(xb + (int64_t)idx * VN);
+        v[u] = load16_stream(xb + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
       }
 #pragma unroll
       for (int u = 0; u < kWideU; ++u) {
