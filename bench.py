@@ -46,7 +46,7 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # algorithmic bytes per fused-classifier call: read the class columns of the logits once and
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
-CE_ROWS_TRAFFIC_BYTES = 1_650_533_000  # measured with rocprofv3 --pmc, see profiles/
+CE_ROWS_TRAFFIC_BYTES = 1_650_508_000  # measured with rocprofv3 --pmc, see profiles/
 
 
 # Kernel durations the per-op rows should agree with: average begin-to-end time of each launch an
@@ -54,42 +54,42 @@ CE_ROWS_TRAFFIC_BYTES = 1_650_533_000  # measured with rocprofv3 --pmc, see prof
 # (same command as this benchmark, under the profiler).  (op, start of config) -> (sum in us, launches)
 KERNEL_TRACE_US = {
     ("layernorm_fwd", "small"): (6.94, "ln_fwd_rows_kernel<2,4>"),
-    ("layernorm_bwd", "small"): (10.05 + 4.38, "ln_bwd_rows_kernel<2,4> + ln_bwd_finalize_kernel"),
-    ("add_layernorm_fwd", "small"): (9.73, "ln_fwd_rows_kernel<2,4,residual>"),
-    ("layernorm_bwd_add", "small"): (16.6 + 4.38, "ln_bwd_rows_kernel<2,3,residual> + ln_bwd_finalize_kernel"),
-    ("layernorm_fwd", "xl"): (19.94, "ln_fwd_rows_kernel<4,2>"),
-    ("layernorm_bwd", "xl"): (30.32 + 4.57, "ln_bwd_rows_kernel<4,2> + ln_bwd_finalize_kernel"),
+    ("layernorm_bwd", "small"): (10.05 + 4.28, "ln_bwd_rows_kernel<2,4> + ln_bwd_finalize_kernel"),
+    ("add_layernorm_fwd", "small"): (10.58, "ln_fwd_rows_kernel<2,4,residual>"),
+    ("layernorm_bwd_add", "small"): (16.13 + 4.28, "ln_bwd_rows_kernel<2,3,residual> + ln_bwd_finalize_kernel"),
+    ("layernorm_fwd", "xl"): (19.85, "ln_fwd_rows_kernel<4,2>"),
+    ("layernorm_bwd", "xl"): (30.24 + 4.56, "ln_bwd_rows_kernel<4,2> + ln_bwd_finalize_kernel"),
     ("add_layernorm_fwd", "xl"): (37.13, "ln_fwd_rows_kernel<4,2,residual>"),
-    ("layernorm_bwd_add", "xl"): (48.81 + 4.57, "ln_bwd_rows_kernel<4,2,residual> + ln_bwd_finalize_kernel"),
-    ("gelu_fwd_tanh", ""): (16.52, "gelu_kernel<tanh,fwd>"),
-    ("gelu_bwd_tanh", ""): (23.69, "gelu_kernel<tanh,bwd>"),
-    ("gelu_fwd_erf", ""): (17.1, "gelu_kernel<erf,fwd>"),
-    ("gelu_bwd_erf", ""): (23.89, "gelu_kernel<erf,bwd>"),
+    ("layernorm_bwd_add", "xl"): (42.19 + 4.56, "ln_bwd_rows_kernel<4,2,residual> + ln_bwd_finalize_kernel"),
+    ("gelu_fwd_tanh", ""): (17.34, "gelu_kernel<tanh,fwd>"),
+    ("gelu_bwd_tanh", ""): (24.34, "gelu_kernel<tanh,bwd>"),
+    ("gelu_fwd_erf", ""): (17.08, "gelu_kernel<erf,fwd>"),
+    ("gelu_bwd_erf", ""): (23.77, "gelu_kernel<erf,bwd>"),
     ("embedding_fwd", "small"): (5.48, "emb_fwd_vec_kernel (uniform and zipf launches averaged)"),
-    ("embedding_bwd", "small"): (17.08 + 6.97 + 4.31, "emb_bwd_rank_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
+    ("embedding_bwd", "small"): (17.03 + 7.03 + 4.31, "emb_bwd_rank_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
     ("embedding_fwd", "xl"): (11.7, "emb_fwd_vec_kernel"),
-    ("embedding_bwd", "xl"): (21.37 + 16.82 + 15.46 + 9.65,
+    ("embedding_bwd", "xl"): (21.42 + 16.78 + 15.56 + 9.66,
                               "emb_bwd_tile_sort_kernel + emb_bwd_merge_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
-    ("adamw_multi_tensor", "small"): (564.21, "adamw_multi_kernel"),
-    ("adamw_multi_tensor", "xl"): (7746.86, "adamw_multi_kernel"),
-    ("adamw_multi_tensor_clipped", "small"): (79.67 + 5.53 + 564.21, "grad_norm_partial_kernel + grad_norm_final_kernel + adamw_multi_kernel"),
-    ("stream_update4", "small"): (589.2, "stream_update4_kernel"),
-    ("stream_update4", "xl"): (7873.78, "stream_update4_kernel"),
-    ("fused_classifier_call", "[8192,50304] bf16, in place"): (4.23 + 282.25 + 4.11, "ce_count_kernel + ce_rows_stream_kernel<7,8> + ce_reduce_kernel"),
-    ("fused_classifier_call", "[8192,50304] bf16, bf16 logits"): (4.32 + 448.49 + 4.35, "ce_count_kernel + ce_rows_stream_kernel<13,4> + ce_reduce_kernel"),
-    ("stream_copy", "25 MB"): (4.94, "stream_copy_kernel<2>"),
-    ("stream_copy", "100 MB"): (17.62, "stream_copy_kernel<2>"),
-    ("stream_copy", "400 MB"): (62.36, "stream_copy_kernel<1>"),
-    ("stream_copy", "1600 MB"): (241.82, "stream_copy_kernel<1>"),
-    ("stream_copy", "3500 MB"): (532.81, "stream_copy_kernel<1>"),
-    ("stream_read", "25 MB"): (5.31, "stream_read_kernel"),
-    ("stream_read", "100 MB"): (16.26, "stream_read_kernel"),
-    ("stream_read", "400 MB"): (60.07, "stream_read_kernel"),
-    ("stream_read", "3500 MB"): (507.0, "stream_read_kernel"),
+    ("adamw_multi_tensor", "small"): (569.0, "adamw_multi_kernel"),
+    ("adamw_multi_tensor", "xl"): (7749.57, "adamw_multi_kernel"),
+    ("adamw_multi_tensor_clipped", "small"): (80.31 + 5.43 + 569.0, "grad_norm_partial_kernel + grad_norm_final_kernel + adamw_multi_kernel"),
+    ("stream_update4", "small"): (587.1, "stream_update4_kernel"),
+    ("stream_update4", "xl"): (7887.86, "stream_update4_kernel"),
+    ("fused_classifier_call", "[8192,50304] bf16, in place"): (4.09 + 280.31 + 4.0, "ce_count_kernel + ce_rows_stream_kernel<7,8> + ce_reduce_kernel"),
+    ("fused_classifier_call", "[8192,50304] bf16, bf16 logits"): (4.24 + 448.81 + 4.35, "ce_count_kernel + ce_rows_stream_kernel<13,4> + ce_reduce_kernel"),
+    ("stream_copy", "25 MB"): (4.95, "stream_copy_kernel<2>"),
+    ("stream_copy", "100 MB"): (17.61, "stream_copy_kernel<2>"),
+    ("stream_copy", "400 MB"): (62.12, "stream_copy_kernel<1>"),
+    ("stream_copy", "1600 MB"): (241.33, "stream_copy_kernel<1>"),
+    ("stream_copy", "3500 MB"): (531.72, "stream_copy_kernel<1>"),
+    ("stream_read", "25 MB"): (5.3, "stream_read_kernel"),
+    ("stream_read", "100 MB"): (16.21, "stream_read_kernel"),
+    ("stream_read", "400 MB"): (59.73, "stream_read_kernel"),
+    ("stream_read", "3500 MB"): (508.39, "stream_read_kernel"),
     ("stream_fill", "25 MB"): (4.93, "stream_fill_kernel"),
-    ("stream_fill", "100 MB"): (17.31, "stream_fill_kernel"),
-    ("stream_fill", "400 MB"): (68.52, "stream_fill_kernel"),
-    ("stream_fill", "3500 MB"): (601.24, "stream_fill_kernel"),
+    ("stream_fill", "100 MB"): (17.17, "stream_fill_kernel"),
+    ("stream_fill", "400 MB"): (69.12, "stream_fill_kernel"),
+    ("stream_fill", "3500 MB"): (605.35, "stream_fill_kernel"),
 }
 
 
