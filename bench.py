@@ -11,14 +11,17 @@ K timed steps between device synchronisations; one JSON line on stdout.
 The same line carries
   roofline      the dominant kernel (the row pass) against the 8 TB/s HBM peak,
                 its duration measured with HIP events inside the timed region
-  per_op        every op of the hot path at its benchmark configuration:
-                ms, GB/s of algorithmic bytes and fraction of the HBM peak,
-                warm (same buffers) and cold (inputs and outputs rotated over
+  per_op        every op of the hot path at its benchmark configuration, one
+                short record each (op, cfg, ms and fraction of the HBM peak per
+                call on cold buffers).  The full table goes to stderr as one
+                JSON line after "[bench-full]" (and to --full-json PATH): ms,
+                GB/s of algorithmic bytes and fraction of the HBM peak, warm
+                (same buffers) and cold (inputs and outputs rotated over
                 > 600 MB so the 256 MB Infinity Cache cannot serve them), each
                 the duration of one call inside a batch of back-to-back calls
-                between one pair of events; next to it the rocprofv3 kernel
-                time the op's launches add up to (kernel_us) and three
-                calibration kernels (plain copy, read only, write only)
+                between one pair of events, and three calibration kernels
+                (plain copy, read only, write only).  The stdout line stays
+                under 8000 bytes
   cpu_baseline  the reference's own op sequence on the ATen CPU backend
                 (oracle/aten_port.py), timed here on this box's host cores
 
@@ -47,61 +50,6 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
 CE_ROWS_TRAFFIC_BYTES = 1_650_508_000  # measured with rocprofv3 --pmc, see profiles/
-
-
-# Kernel durations the per-op rows should agree with: average begin-to-end time of each launch an
-# op makes, from the rocprofv3 kernel trace summarised in profiles/bench_all_ops_kernel_trace.txt
-# (same command as this benchmark, under the profiler).  (op, start of config) -> (sum in us, launches)
-KERNEL_TRACE_US = {
-    ("layernorm_fwd", "small"): (6.94, "ln_fwd_rows_kernel<2,4>"),
-    ("layernorm_bwd", "small"): (10.05 + 4.28, "ln_bwd_rows_kernel<2,4> + ln_bwd_finalize_kernel"),
-    ("add_layernorm_fwd", "small"): (10.58, "ln_fwd_rows_kernel<2,4,residual>"),
-    ("layernorm_bwd_add", "small"): (16.13 + 4.28, "ln_bwd_rows_kernel<2,3,residual> + ln_bwd_finalize_kernel"),
-    ("layernorm_fwd", "xl"): (19.85, "ln_fwd_rows_kernel<4,2>"),
-    ("layernorm_bwd", "xl"): (30.24 + 4.56, "ln_bwd_rows_kernel<4,2> + ln_bwd_finalize_kernel"),
-    ("add_layernorm_fwd", "xl"): (37.13, "ln_fwd_rows_kernel<4,2,residual>"),
-    ("layernorm_bwd_add", "xl"): (42.19 + 4.56, "ln_bwd_rows_kernel<4,2,residual> + ln_bwd_finalize_kernel"),
-    ("gelu_fwd_tanh", ""): (17.34, "gelu_kernel<tanh,fwd>"),
-    ("gelu_bwd_tanh", ""): (24.34, "gelu_kernel<tanh,bwd>"),
-    ("gelu_fwd_erf", ""): (17.08, "gelu_kernel<erf,fwd>"),
-    ("gelu_bwd_erf", ""): (23.77, "gelu_kernel<erf,bwd>"),
-    ("embedding_fwd", "small"): (5.48, "emb_fwd_vec_kernel (uniform and zipf launches averaged)"),
-    ("embedding_bwd", "small"): (17.03 + 7.03 + 4.31, "emb_bwd_rank_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
-    ("embedding_fwd", "xl"): (11.7, "emb_fwd_vec_kernel"),
-    ("embedding_bwd", "xl"): (21.42 + 16.78 + 15.56 + 9.66,
-                              "emb_bwd_tile_sort_kernel + emb_bwd_merge_kernel + emb_bwd_reduce_kernel + emb_bwd_finish_kernel"),
-    ("adamw_multi_tensor", "small"): (569.0, "adamw_multi_kernel"),
-    ("adamw_multi_tensor", "xl"): (7749.57, "adamw_multi_kernel"),
-    ("adamw_multi_tensor_clipped", "small"): (80.31 + 5.43 + 569.0, "grad_norm_partial_kernel + grad_norm_final_kernel + adamw_multi_kernel"),
-    ("stream_update4", "small"): (587.1, "stream_update4_kernel"),
-    ("stream_update4", "xl"): (7887.86, "stream_update4_kernel"),
-    ("fused_classifier_call", "[8192,50304] bf16, in place"): (4.09 + 280.31 + 4.0, "ce_count_kernel + ce_rows_stream_kernel<7,8> + ce_reduce_kernel"),
-    ("fused_classifier_call", "[8192,50304] bf16, bf16 logits"): (4.24 + 448.81 + 4.35, "ce_count_kernel + ce_rows_stream_kernel<13,4> + ce_reduce_kernel"),
-    ("stream_copy", "25 MB"): (4.95, "stream_copy_kernel<2>"),
-    ("stream_copy", "100 MB"): (17.61, "stream_copy_kernel<2>"),
-    ("stream_copy", "400 MB"): (62.12, "stream_copy_kernel<1>"),
-    ("stream_copy", "1600 MB"): (241.33, "stream_copy_kernel<1>"),
-    ("stream_copy", "3500 MB"): (531.72, "stream_copy_kernel<1>"),
-    ("stream_read", "25 MB"): (5.3, "stream_read_kernel"),
-    ("stream_read", "100 MB"): (16.21, "stream_read_kernel"),
-    ("stream_read", "400 MB"): (59.73, "stream_read_kernel"),
-    ("stream_read", "3500 MB"): (508.39, "stream_read_kernel"),
-    ("stream_fill", "25 MB"): (4.93, "stream_fill_kernel"),
-    ("stream_fill", "100 MB"): (17.17, "stream_fill_kernel"),
-    ("stream_fill", "400 MB"): (69.12, "stream_fill_kernel"),
-    ("stream_fill", "3500 MB"): (605.35, "stream_fill_kernel"),
-}
-
-
-def attach_kernel_trace(rec):
-    """Adds the profiled kernel time an op's launches add up to, for cross-checking ms_cold."""
-    for (op, prefix), (us, launches) in KERNEL_TRACE_US.items():
-        if rec["op"] == op and rec["config"].startswith(prefix):
-            rec["kernel_us"] = round(us, 2)
-            rec["kernel_launches"] = launches
-            rec["ms_cold_over_kernel"] = round(rec["ms_cold"] * 1e3 / us, 3)
-            return rec
-    return rec
 
 
 def log(*a):
@@ -747,6 +695,7 @@ def main():
     ap.add_argument("--no-xl-ce", dest="xl_ce", action="store_false")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="K",
                     help="also run K plain 1 GiB copies (to scale hardware traffic counters)")
+    ap.add_argument("--full-json", default="", metavar="PATH", help="also write the full per-op table to this file")
     ap.add_argument("--cpu-rows", type=int, default=CE_N)
     ap.add_argument("--cpu-reps", type=int, default=5)
     args = ap.parse_args()
@@ -790,11 +739,35 @@ def main():
         if table:
             cpu_per_op(args, torch, table)
 
+    line = result_line(args, head, value, achieved, cpu, table)
+    full = dict(line, per_op=table)
+    log("[bench-full] " + json.dumps(full))
+    if args.full_json:
+        with open(args.full_json, "w") as f:
+            json.dump(full, f, indent=1)
+    print(json.dumps(line), flush=True)
+
+
+MAX_LINE_BYTES = 8000  # the result line on stdout stays below this; the full table goes to stderr
+
+
+def compact_per_op(table):
+    """One short record per row of the per-op table: op, configuration tag, cold ms per call,
+    cold fraction of the HBM peak.  Everything else a row carries is in the full table."""
+    out = []
     for rec in table:
-        attach_kernel_trace(rec)
+        cfg = rec["config"].split(",")[0].split(":")[0]
+        out.append({"op": rec["op"], "cfg": cfg[:40], "ms": rec["ms_cold"], "frac": rec["frac_cold"]})
+    return out
+
+
+def result_line(args, head, value, achieved, cpu, table):
+    """The one JSON line for stdout.  `per_op` is compact and comes before `roofline` and
+    `cpu_baseline`, so the end of the line always shows those two."""
     line = {
         "metric": "per-op HBM GB/s (% of MI355X peak); fused CE ms at 8192x50257 bf16",
-        "metric_note": "value = the fused classifier's whole-step GB/s (the ms is ms_per_step); every other op is in per_op",
+        "metric_note": "value = the fused classifier's whole-step GB/s (the ms is ms_per_step); every other op is in per_op "
+                       "(ms and fraction of the HBM peak per call, cold buffers); the full table is on stderr after [bench-full]",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -813,6 +786,7 @@ def main():
             "logits_buffers_rotated": head["buffers"],
             "loss": round(head["loss"], 5),
         },
+        "per_op": compact_per_op(table),
         "roofline": {
             "bound": "hbm",
             "kernel": "ce_rows_stream_kernel<bf16_t, bf16_t, 7, 8>",
@@ -828,9 +802,13 @@ def main():
             "traffic_over_algorithmic": round(CE_ROWS_TRAFFIC_BYTES / CE_BYTES, 4),
         },
         "cpu_baseline": cpu,
-        "per_op": table,
     }
-    print(json.dumps(line), flush=True)
+    # the calibration rows go first if the line ever has to shrink
+    while len(json.dumps(line)) > MAX_LINE_BYTES and line["per_op"]:
+        drop = next((i for i, r in enumerate(line["per_op"]) if r["op"].startswith("stream_")), len(line["per_op"]) - 1)
+        line["per_op"].pop(drop)
+        line["per_op_truncated"] = True
+    return line
 
 
 if __name__ == "__main__":
