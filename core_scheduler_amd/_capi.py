@@ -89,6 +89,11 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
     ),
+    "cs_layernorm_backward_rows_pending": (
+        c_int,
+        [c_void_p] * 8 + [c_size_t, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int64] + [c_int] * 4
+        + [c_void_p],
+    ),
     "cs_layernorm_backward": (
         c_int,
         [c_void_p] * 9 + [c_size_t, c_int64, c_int64] + [c_int] * 5 + [c_void_p],

@@ -209,6 +209,15 @@ __device__ __forceinline__ A block_reduce(A v, Op op, A identity, A *scratch) {
   return r;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a workgroup-scope fence,
+// for which the compiler waits until every global store the wave has issued is acknowledged
+// (s_waitcnt vmcnt(0)): behind a row's worth of streaming stores that is one to two microseconds.
+// Here a wave only waits for its own LDS accesses before it joins the barrier.  Use it where the
+// data exchanged between the waves lives in the LDS and nowhere else.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ------------------------------------------------------------ host side
 inline int launch_status() {
   const hipError_t e = hipGetLastError();

@@ -26,6 +26,7 @@
 
 #include <math.h>
 
+#include <atomic>
 #include <type_traits>
 
 // Every product and sum below is rounded as written: no multiply-add contraction, so that the
@@ -315,6 +316,66 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
   }
 }
 
+// ------------------------------------------------- column sums of partial rows
+// What a launch of the row kernel may do on the side: the column sums of an EARLIER call's partial
+// rows (written by a launch that is complete when this one starts).  The first `blocks`
+// workgroups of the grid do that and leave; the row work starts at workgroup `blocks`.
+struct LnPending {
+  const float *partial;  // nullptr: nothing pending
+  void *dgamma, *dbeta;  // of the earlier call; either may be nullptr
+  int nparts, accumulate, blocks;
+};
+
+// Adds `nparts` partial rows in a fixed order.  Partial rows are permuted: position
+// p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  One tile = 32 positions of dgamma or
+// dbeta: thread (cx, ry) of 32 x 16 sums partial rows ry, ry+16, ... for one position, sixteen
+// loads in flight and none of them under a condition (this work waits for a row kernel and is all
+// latency), then row 0 adds the 16 sub-sums in order.  `sub` is 16 x 32 floats of LDS.
+constexpr int kLnFinCols = 32, kLnFinRows = 16, kLnFinInFlight = 16;
+
+template <typename TP, int THREADS = kLnFinCols * kLnFinRows>
+__device__ __forceinline__ void ln_finalize_tile(const float *__restrict__ partial, int nparts, TP *__restrict__ out,
+                                                 int which, int tile, int C, int vn, int accumulate, float *sub,
+                                                 int tid) {
+  static_assert(THREADS >= kLnFinCols * kLnFinRows, "a tile takes 512 threads; further ones only join the barrier");
+  const int cx = tid % kLnFinCols, ry = tid / kLnFinCols;
+  const int col = tile * kLnFinCols + cx;  // a position in the permuted row
+  float s = 0.f;
+  if (col < C && ry < kLnFinRows) {
+    const float *src = partial + (int64_t)which * C + col;
+    const int64_t stride = 2 * (int64_t)C;
+    for (int p0 = ry; p0 < nparts; p0 += kLnFinRows * kLnFinInFlight) {
+      float v[kLnFinInFlight];
+#pragma unroll
+      for (int u = 0; u < kLnFinInFlight; ++u) {
+        const int p = p0 + u * kLnFinRows;
+        v[u] = src[(int64_t)(p < nparts ? p : nparts - 1) * stride];
+      }
+#pragma unroll
+      for (int u = 0; u < kLnFinInFlight; ++u) s += p0 + u * kLnFinRows < nparts ? v[u] : 0.f;
+    }
+  }
+  if (ry < kLnFinRows) sub[ry * kLnFinCols + cx] = s;
+  __syncthreads();
+  if (ry == 0 && col < C) {
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < kLnFinRows; ++r) t += sub[r * kLnFinCols + cx];
+    const int nvec = C / vn;
+    const int real = (col % nvec) * vn + col / nvec;  // the column this position stands for
+    if (accumulate) t += to_acc(out[real]);
+    out[real] = from_acc<TP>(t);
+  }
+}
+// workgroup b of the 2 * ceil(C/32) that cover a pending call: even b dgamma, odd b dbeta
+template <typename TP, int THREADS = kLnFinCols * kLnFinRows>
+__device__ __forceinline__ void ln_finalize_pending(const LnPending &pend, int b, int C, int vn, float *sub, int tid) {
+  const int which = b & 1;
+  TP *out = (TP *)(which == 0 ? pend.dgamma : pend.dbeta);
+  if (out == nullptr) return;  // block-uniform
+  ln_finalize_tile<TP, THREADS>(pend.partial, pend.nparts, out, which, b >> 1, C, vn, pend.accumulate, sub, tid);
+}
+
 // ----------------------------------------------------------- fast backward
 // One wave per row, the row (dy and x) in registers, gamma and the per-column partial sums in
 // registers for all rows a wave visits (rows gw, gw + n_waves, ...).  No software prefetch:
@@ -333,14 +394,20 @@ template <typename TDY, typename TX, typename TDX, typename TP, int VPL, int WPE
           bool HAS_DP, bool HAS_DRES>
 __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
     const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
-    const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *__restrict__ dx,
-    float *__restrict__ partial, int64_t rows, int C, const TDX *__restrict__ dres) {
+    const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *dx,
+    float *__restrict__ partial, int64_t rows, int C, const TDX *dres /* dx may be dres */,
+    const LnPending pend) {
   constexpr int VN = Vec16<TX>::n;
-  extern __shared__ float lds[];  // [waves per block][C]
+  extern __shared__ float lds[];  // [waves per block][C], at least 16 x 32 floats with pending sums
+  if ((int)blockIdx.x < pend.blocks) {
+    ln_finalize_pending<TP>(pend, blockIdx.x, C, VN, lds, threadIdx.x);
+    return;
+  }
+  const int bid = blockIdx.x - pend.blocks;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   constexpr int kWaves = kLnBwdThreads / kWave;
-  const int64_t step = (int64_t)gridDim.x * kWaves;
+  const int64_t step = (int64_t)(gridDim.x - pend.blocks) * kWaves;
   const int nvec = C / VN;
   const float inv_c = 1.0f / (float)C;
 
@@ -356,7 +423,7 @@ __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
     if (HAS_DX && lane + kWave * j < nvec) load_n<TP, VN>(gamma + (lane + kWave * j) * VN, g[j]);
   }
 
-  for (int64_t row = (int64_t)blockIdx.x * kWaves + wave; row < rows; row += step) {
+  for (int64_t row = (int64_t)bid * kWaves + wave; row < rows; row += step) {
     RowSet<TDY, VN, VPL, 1> dcur;
     RowSet<TX, VN, VPL, 1> xcur;
     RowSet<TDX, VN, VPL, 1> rcur;  // this row of dresidual, in flight during the reductions
@@ -444,9 +511,232 @@ __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) s += lds[w * C + c];
-        partial[((int64_t)blockIdx.x * 2 + which) * C + c] = s;
+        partial[((int64_t)bid * 2 + which) * C + c] = s;
       }
       __syncthreads();
+    }
+  }
+}
+
+// --------------------------------- rows on whole waves or on halves of a wave
+// LPR lanes per row: 64 (a wave per row) or 32: two rows per wave, side by side, lanes 0-31 on row
+// 2p, lanes 32-63 on row 2p + 1, for rows of at most 32 * VPL vectors.  A 768-column row of 16-bit
+// data is 96 vectors = 32 lanes x 3, so every lane slot is used (on whole waves it takes two
+// vectors per lane and leaves a quarter of them empty), a wave finishes two rows per round trip to
+// memory, and the same number of waves leaves half as many rows behind them.  The two row sums
+// are reduced per half; the column sums of the halves meet in the LDS fold at the end.
+constexpr int kHalf = kWave / 2;
+
+// Sum over the LPR lanes that share a row (all 64, or each half of the wave on its own).
+template <int LPR>
+__device__ __forceinline__ float row_lanes_sum(float v, bool upper) {
+  v += dpp_f32<kDppQuadXor1>(v);
+  v += dpp_f32<kDppQuadXor2>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppRowMirror>(v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  if constexpr (LPR == kWave) return (r0 + r1) + (r2 + r3);
+  return upper ? r2 + r3 : r0 + r1;
+}
+
+template <typename T, int VN, int VPL>
+struct Strip {
+  Raw<T, VN> v[VPL];
+};
+// every lane loads (from the last vector of the row again where it has none of its own)
+template <typename T, int VN, int VPL, int LPR>
+__device__ __forceinline__ void load_strip(Strip<T, VN, VPL> &dst, const T *src, int64_t row, int C, int nvec,
+                                           int hl) {
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int idx = hl + LPR * j;
+    dst.v[j] = load_raw<T, VN>(src + row * C + (int64_t)(idx < nvec ? idx : nvec - 1) * VN);
+  }
+}
+template <typename T, int VN, int VPL, int LPR>
+__device__ __forceinline__ void zero_strip_unless(Strip<T, VN, VPL> &r, bool row_ok, int nvec, int hl) {
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const bool keep = row_ok && hl + LPR * j < nvec;
+#pragma unroll
+    for (int q = 0; q < VN / Vec16<T>::n; ++q) {
+      u32x4 w = __builtin_bit_cast(u32x4, r.v[j].v[q]);
+      w.x = keep ? w.x : 0u;
+      w.y = keep ? w.y : 0u;
+      w.z = keep ? w.z : 0u;
+      w.w = keep ? w.w : 0u;
+      r.v[j].v[q] = __builtin_bit_cast(Vec16<T>, w);
+    }
+  }
+}
+
+#ifndef CS_LN_PAIR_FOLD
+#define CS_LN_PAIR_FOLD 1
+#endif
+
+// PF: the next step's rows are requested before the current ones are worked on.
+// KEEP: x-hat and dy*gamma stay unpacked across the two row sums instead of being unpacked and
+// normalised again for the second pass (at 16-bit storage the kernel is as close to the VALU
+// limit as to the memory's); takes VPL * 2 * VN more registers.
+template <typename TDY, typename TX, typename TDX, typename TP, int THREADS, int LPR, int VPL, int WPE, bool PF,
+          bool KEEP,
+          bool HAS_DX, bool HAS_DP, bool HAS_DRES>
+__global__ __launch_bounds__(THREADS, WPE) void ln_bwd_kernel(
+    const TDY *__restrict__ dy, const TX *__restrict__ x, const float *__restrict__ mean,
+    const float *__restrict__ rstd, const TP *__restrict__ gamma, TDX *dx /* may be dres */,
+    float *__restrict__ partial, int64_t rows, int C, const TDX *dres, const LnPending pend) {
+  constexpr int VN = Vec16<TX>::n;
+  constexpr int RPW = kWave / LPR;  // rows a wave works on side by side
+  extern __shared__ float lds[];    // [RPW * waves per block][C], at least 16 x 32 floats
+  if ((int)blockIdx.x < pend.blocks) {
+    ln_finalize_pending<TP, THREADS>(pend, blockIdx.x, C, VN, lds, threadIdx.x);
+    return;
+  }
+  const int bid = blockIdx.x - pend.blocks, nblocks = gridDim.x - pend.blocks;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const bool upper = LPR == kHalf && lane >= kHalf;
+  const int hl = lane & (LPR - 1);
+  constexpr int kWaves = THREADS / kWave;
+  const int64_t step = (int64_t)nblocks * kWaves;
+  const int64_t nsteps = (rows + RPW - 1) / RPW;  // row groups: one per wave and step
+  const int nvec = C / VN;
+  const float inv_c = 1.0f / (float)C;
+
+  float acc_g[VPL][VN], acc_b[VPL][VN], g[VPL][VN];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int idx = hl + LPR * j;
+#pragma unroll
+    for (int k = 0; k < VN; ++k) {
+      acc_g[j][k] = 0.f;
+      acc_b[j][k] = 0.f;
+    }
+    if constexpr (HAS_DX) load_n<TP, VN>(gamma + (idx < nvec ? idx : nvec - 1) * VN, g[j]);
+  }
+
+  Strip<TDY, VN, VPL> dcur, dnxt;
+  Strip<TX, VN, VPL> xcur, xnxt;
+  Strip<TDX, VN, VPL> rcur, rnxt;  // this row of dresidual, in flight during the reductions
+  float mu = 0.f, rs = 0.f, nmu = 0.f, nrs = 0.f;
+  int64_t p = (int64_t)bid * kWaves + wave;
+  auto issue = [&](int64_t p_, Strip<TDY, VN, VPL> &d, Strip<TX, VN, VPL> &xx, Strip<TDX, VN, VPL> &rr, float &m_,
+                   float &r_) {
+    const int64_t row = RPW * p_ + (upper ? 1 : 0);
+    const int64_t rowc = row < rows ? row : rows - 1;
+    load_strip<TDY, VN, VPL, LPR>(d, dy, rowc, C, nvec, hl);
+    load_strip<TX, VN, VPL, LPR>(xx, x, rowc, C, nvec, hl);
+    if constexpr (HAS_DRES) load_strip<TDX, VN, VPL, LPR>(rr, dres, rowc, C, nvec, hl);
+    m_ = mean[rowc];
+    r_ = rstd[rowc];
+  };
+  if constexpr (PF) {
+    if (p < nsteps) issue(p, dcur, xcur, rcur, mu, rs);
+  }
+  for (; p < nsteps; p += step) {
+    if constexpr (PF) {
+      if (p + step < nsteps) issue(p + step, dnxt, xnxt, rnxt, nmu, nrs);
+    } else {
+      issue(p, dcur, xcur, rcur, mu, rs);
+    }
+    const int64_t row = RPW * p + (upper ? 1 : 0);
+    const bool row_ok = row < rows;
+    zero_strip_unless<TDY, VN, VPL, LPR>(dcur, row_ok, nvec, hl);  // lanes without data add nothing below
+    float s1 = 0.f, s2 = 0.f;
+    float xh[KEEP ? VPL : 1][VN], gd[KEEP ? VPL : 1][VN];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int jj = KEEP ? j : 0;
+#pragma unroll
+      for (int k = 0; k < VN; ++k) {
+        xh[jj][k] = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
+        const float dv = raw_get<TDY, VN>(dcur.v[j], k);
+        if constexpr (HAS_DP) {
+          acc_g[j][k] = __builtin_fmaf(dv, xh[jj][k], acc_g[j][k]);
+          acc_b[j][k] += dv;
+        }
+        if constexpr (HAS_DX) {
+          gd[jj][k] = dv * g[j][k];
+          s1 += gd[jj][k];
+          s2 = __builtin_fmaf(gd[jj][k], xh[jj][k], s2);
+        }
+      }
+    }
+    if constexpr (HAS_DX) {
+      // rstd * (dy gamma - mean(dy gamma) - xhat mean(dy gamma xhat)) with the row's three
+      // factors folded first: two operations per element
+      const float cb = -(row_lanes_sum<LPR>(s1, upper) * inv_c) * rs;
+      const float cc = -(row_lanes_sum<LPR>(s2, upper) * inv_c) * rs;
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int jj = KEEP ? j : 0;
+        if constexpr (!KEEP) {
+          // unpacked again from the packed row rather than kept as floats across the reduction
+          forget_unpacked(xcur.v[j]);
+          forget_unpacked(dcur.v[j]);
+        }
+        if constexpr (HAS_DRES) forget_unpacked(rcur.v[j]);  // keeps its load where it was issued
+        const int idx = hl + LPR * j;
+        float o[VN];
+#pragma unroll
+        for (int k = 0; k < VN; ++k) {
+          if constexpr (!KEEP) {
+            xh[jj][k] = (raw_get<TX, VN>(xcur.v[j], k) - mu) * rs;
+            gd[jj][k] = raw_get<TDY, VN>(dcur.v[j], k) * g[j][k];
+          }
+          o[k] = __builtin_fmaf(xh[jj][k], cc, __builtin_fmaf(gd[jj][k], rs, cb));
+          if constexpr (HAS_DRES) o[k] = round_through<TDX>(o[k]) + raw_get<TDX, VN>(rcur.v[j], k);
+        }
+        if (row_ok && idx < nvec) store_n<TDX, VN>(dx + row * C + (int64_t)idx * VN, o);
+      }
+    }
+    if constexpr (PF) {
+      dcur = dnxt;
+      xcur = xnxt;
+      if constexpr (HAS_DRES) rcur = rnxt;
+      mu = nmu;
+      rs = nrs;
+    }
+  }
+
+#if CS_LN_PAIR_FOLD <= 0
+  if constexpr (HAS_DP) {
+    float t = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+#pragma unroll
+      for (int k = 0; k < VN; ++k) t += acc_g[j][k] * acc_b[j][k];
+    if (t == 12345.678f) partial[threadIdx.x] = t;
+  }
+#endif
+  if constexpr (HAS_DP && CS_LN_PAIR_FOLD > 0) {
+    // Fold the block's waves (half-waves), dgamma first, then dbeta through the same LDS.  Column
+    // idx*VN + k is kept at position k*nvec + idx, in the LDS and in the partial rows: lanes
+    // then write consecutive words (no bank conflicts); the finalize step undoes the permutation.
+    // (Measured against 16-byte LDS writes in a layout that suits them, with 16-byte or 4-byte
+    // reads: 0.3-0.9 us slower per launch at [8192,768] than these 4-byte accesses.)
+    const int hw = wave * RPW + (upper ? 1 : 0);
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) {
+        const int idx = hl + LPR * j;
+        if (idx < nvec) {
+#pragma unroll
+          for (int k = 0; k < VN; ++k) lds[hw * C + k * nvec + idx] = which == 0 ? acc_g[j][k] : acc_b[j][k];
+        }
+      }
+      lds_barrier();
+      for (int c = threadIdx.x; c < C; c += THREADS) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < RPW * kWaves; ++w) s += lds[w * C + c];
+        partial[((int64_t)bid * 2 + which) * C + c] = s;
+      }
+      if (which == 0) lds_barrier();
     }
   }
 }
@@ -610,49 +900,16 @@ __global__ __launch_bounds__(kLnBwdThreads) void ln_bwd_split_rows_kernel(
   }
 }
 
-// Adds `nparts` partial rows in a fixed order.  Partial rows are permuted: position
-// p = k*nvec + idx holds column idx*vn + k (nvec = C/vn).  grid (ceil(C/32), 2), block
-// (32, 32): thread (cx, ry) sums partial rows ry, ry+32, ... for one column, sixteen loads in
-// flight and none of them under a condition (this launch waits for the row kernel and is all
-// latency: with 512 partial rows a thread makes one round trip), then row 0 of the block adds
-// the 32 sub-sums in order.
-constexpr int kLnFinCols = 32, kLnFinRows = 32, kLnFinInFlight = 16;
-
+// The column sums as a launch of their own: grid 2 * ceil(C/32) workgroups of 32 x 16 threads, even
+// ones dgamma, odd ones dbeta (the same tiles, in the same order of additions, as the pending
+// form inside the row kernel's launch).
 template <typename TP>
 __global__ __launch_bounds__(kLnFinCols *kLnFinRows) void ln_bwd_finalize_kernel(
     const float *__restrict__ partial, int nparts, TP *__restrict__ dgamma, TP *__restrict__ dbeta,
     int C, int vn, int accumulate) {
-  __shared__ float sub[kLnFinRows][kLnFinCols];
-  const int which = blockIdx.y;
-  TP *out = which == 0 ? dgamma : dbeta;
-  if (out == nullptr) return;  // block-uniform
-  const int col = blockIdx.x * kLnFinCols + threadIdx.x;  // a position in the permuted row
-  float s = 0.f;
-  if (col < C) {
-    const float *src = partial + (int64_t)which * C + col;
-    const int64_t stride = 2 * (int64_t)C;
-    for (int p0 = threadIdx.y; p0 < nparts; p0 += kLnFinRows * kLnFinInFlight) {
-      float v[kLnFinInFlight];
-#pragma unroll
-      for (int u = 0; u < kLnFinInFlight; ++u) {
-        const int p = p0 + u * kLnFinRows;
-        v[u] = src[(int64_t)(p < nparts ? p : nparts - 1) * stride];
-      }
-#pragma unroll
-      for (int u = 0; u < kLnFinInFlight; ++u) s += p0 + u * kLnFinRows < nparts ? v[u] : 0.f;
-    }
-  }
-  sub[threadIdx.y][threadIdx.x] = s;
-  __syncthreads();
-  if (threadIdx.y == 0 && col < C) {
-    float t = 0.f;
-#pragma unroll
-    for (int r = 0; r < kLnFinRows; ++r) t += sub[r][threadIdx.x];
-    const int nvec = C / vn;
-    const int real = (col % nvec) * vn + col / nvec;  // the column this position stands for
-    if (accumulate) t += to_acc(out[real]);
-    out[real] = from_acc<TP>(t);
-  }
+  __shared__ float sub[kLnFinRows * kLnFinCols];
+  const LnPending pend{partial, dgamma, dbeta, nparts, accumulate, (int)gridDim.x};
+  ln_finalize_pending<TP>(pend, blockIdx.x, C, vn, sub, threadIdx.x);
 }
 
 // ------------------------------------------------------ elementwise add
@@ -913,97 +1170,251 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   return launch_status();
 }
 
-// Partial rows [2C fp32 each] that the row kernel of a plan leaves for the finalize kernel.
-int bwd_partial_rows(int64_t rows, int vpl) {
-  // the wide plan with parameter gradients: two waves per row, so half as many rows per workgroup
-  if (vpl == 8) return ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
-  return ln_blocks(rows, 1, vpl <= 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
+// ---- backward plans.  Which row kernel takes a shape, with what launch: one function, used by
+// the launches, the workspace sizes and the partial-row counts alike.
+#ifndef CS_LN_PAIRS
+#define CS_LN_PAIRS 1
+#endif
+#ifndef CS_LN_PAIR_PF
+#define CS_LN_PAIR_PF false
+#endif
+#ifndef CS_LN_PAIR_KEEP
+#define CS_LN_PAIR_KEEP true
+#endif
+#ifndef CS_LN_PAIR_MAX_BLOCKS
+#define CS_LN_PAIR_MAX_BLOCKS 256
+#endif
+// Rows of 4 vectors per lane (the 1600-column row at 16 bit) on ln_bwd_kernel, a wave per row:
+// 0 never, 1 when only dgamma/dbeta are asked for, 2 always.  Measured at [16384,1600] bf16 with
+// 512 threads, against ln_bwd_rows_kernel: dgamma/dbeta alone 22.4 against 45.8 us (every lane
+// loads: nothing serialises the loads), dx alone 29.0 against 28.4 us, all three 33.3 against
+// 33.7 us; with the next row prefetched, or 1024 threads, the kernel spills.  The two kernels give
+// the same partial rows bit for bit (same rows per wave, same order of additions).
+#ifndef CS_LN_W4_NEW
+#define CS_LN_W4_NEW 1
+#endif
+#ifndef CS_LN_W4_THREADS
+#define CS_LN_W4_THREADS 512
+#endif
+#ifndef CS_LN_W4_WPE
+#define CS_LN_W4_WPE 2
+#endif
+#ifndef CS_LN_W4_PF
+#define CS_LN_W4_PF false
+#endif
+#ifndef CS_LN_W4_KEEP
+#define CS_LN_W4_KEEP false
+#endif
+enum BwdKind {
+  kBwdNone = 0,  // no row-in-registers plan: the general kernels
+  kBwdHalf1,     // ln_bwd_kernel, two rows per wave, 1 vector per lane (rows of up to 32 vectors)
+  kBwdHalf3,     // ln_bwd_kernel, two rows per wave, 3 vectors per lane (65 to 96 vectors: C = 768 at 16 bit)
+  kBwdWave4,     // ln_bwd_kernel, a wave per row, 4 vectors per lane
+  kBwdRows,      // ln_bwd_rows_kernel, 1 / 2 / 4 / 8 (no parameter gradients) vectors per lane
+  kBwdSplit,     // ln_bwd_split_rows_kernel: 8 vectors per lane with parameter gradients
+};
+struct BwdPlan {
+  BwdKind kind = kBwdNone;
+  int vpl = 0;
+  int threads = kLnBwdThreads;
+  int blocks = 0;         // workgroups of row work = partial rows left behind when dgamma/dbeta are wanted
+  size_t fold_lds = 0;    // LDS of the column-sum fold
+};
+constexpr int kLnMaxPartialRows = 512;
+static_assert(kLnBwdMaxBlocksNarrow <= kLnMaxPartialRows && kLnBwdMaxBlocks <= kLnMaxPartialRows &&
+                  CS_LN_PAIR_MAX_BLOCKS <= kLnMaxPartialRows,
+              "every plan's grid cap fits the finalize step's row limit");
+
+BwdPlan bwd_plan(int64_t rows, int64_t C, int x_dtype, bool want_dp, bool want_dx = true) {
+  BwdPlan b;
+  const FastPlan p = fast_plan(C, x_dtype);
+  if (p.vpl == 0) return b;
+  const int vn = 16 / (int)dtype_size(x_dtype);
+  const int64_t nvec = C / vn;
+  b.vpl = p.vpl;
+  if (CS_LN_PAIRS && (nvec <= kHalf || (nvec > kWave && nvec <= 3 * kHalf))) {
+    b.kind = nvec <= kHalf ? kBwdHalf1 : kBwdHalf3;
+    b.vpl = nvec <= kHalf ? 1 : 3;
+    const int64_t n = ceil_div((rows + 1) / 2, (int64_t)(kLnBwdThreads / kWave));
+    b.blocks = (int)(n < CS_LN_PAIR_MAX_BLOCKS ? n : CS_LN_PAIR_MAX_BLOCKS);
+    b.fold_lds = (size_t)(kLnBwdThreads / kWave) * 2 * C * sizeof(float);
+  } else if (p.vpl == 4 && (CS_LN_W4_NEW == 2 || (CS_LN_W4_NEW == 1 && !want_dx))) {
+    b.kind = kBwdWave4;
+    b.threads = CS_LN_W4_THREADS;
+    b.blocks = ln_blocks(rows, 1, kLnBwdMaxBlocks, b.threads);
+    b.fold_lds = (size_t)(b.threads / kWave) * C * sizeof(float);
+  } else if (p.vpl == 8 && want_dp) {
+    // with the dgamma/dbeta accumulators a row no longer fits one wave's registers (a single-wave
+    // kernel spilled ~1 KB per lane), so two waves share each row
+    b.kind = kBwdSplit;
+    b.blocks = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
+    b.fold_lds = (size_t)(kLnBwdThreads / kWave / 2) * 4 * kWave * vn * sizeof(float);
+  } else {
+    b.kind = kBwdRows;
+    b.blocks = ln_blocks(rows, 1, p.vpl <= 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
+    b.fold_lds = (size_t)(kLnBwdThreads / kWave) * C * sizeof(float);
+  }
+  return b;
 }
 
+// Column order inside a partial row, as the `vn` of ln_finalize_tile: every row kernel leaves
+// column idx*vn + k at position k*(C/vn) + idx.
+int partial_vn(int x_dtype) { return 16 / (int)dtype_size(x_dtype); }
+
 enum BwdPhase { kBwdWhole = 0, kBwdRowsOnly = 1 };
+
+// An earlier call's partial rows whose column sums ride in this call's launch (host side of
+// LnPending); partial == nullptr: none.
+struct PendingSums {
+  const void *partial = nullptr;
+  int64_t nparts = 0;
+  void *dgamma = nullptr, *dbeta = nullptr;
+  int accumulate = 0;
+};
+
+template <typename TP>
+int launch_finalize(const void *partial, int64_t nparts, void *dgamma, void *dbeta, int64_t C, int vn,
+                    int accumulate, hipStream_t s) {
+  ln_bwd_finalize_kernel<TP><<<dim3(2 * (unsigned)ceil_div(C, (int64_t)kLnFinCols)), dim3(kLnFinCols * kLnFinRows), 0, s>>>(
+      (const float *)partial, (int)nparts, (TP *)dgamma, (TP *)dbeta, (int)C, vn, accumulate);
+  return launch_status();
+}
+
+// A launch may ask for more dynamic LDS than the 64 KB it gets by default once the kernel's limit
+// has been raised; once per kernel and device.
+template <typename K>
+int allow_lds(K kernel, size_t bytes, size_t most, std::atomic<bool> *done) {
+  if (bytes <= 64 * 1024) return CS_OK;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  if (!done[dev].load(std::memory_order_acquire)) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
+    if (e != hipSuccess) return (int)e;
+    done[dev].store(true, std::memory_order_release);
+  }
+  return CS_OK;
+}
+
+template <typename TDY, typename TX, typename TDX, typename TP, int THREADS, int LPR, int VPL, int WPE, bool PF,
+          bool KEEP, bool HAS_DX, bool HAS_DP, bool HAS_DRES>
+int launch_bwd_kernel(const void *dy, const void *x, const void *mean, const void *rstd, const void *gamma,
+                      void *dx, void *workspace, int64_t rows, int64_t C, const void *dres, const LnPending &pend,
+                      int blocks, size_t lds, hipStream_t s) {
+  static std::atomic<bool> lds_allowed[64];
+  auto kernel = ln_bwd_kernel<TDY, TX, TDX, TP, THREADS, LPR, VPL, WPE, PF, KEEP, HAS_DX, HAS_DP, HAS_DRES>;
+  // the fold of the widest row this instantiation takes: [rows side by side x waves][C] floats
+  constexpr size_t kMostLds = (size_t)THREADS * VPL * Vec16<TX>::n * sizeof(float);
+  const int st = allow_lds(kernel, lds, kMostLds, lds_allowed);
+  if (st != CS_OK) return st;
+  kernel<<<dim3((unsigned)(blocks + pend.blocks)), dim3(THREADS), lds, s>>>(
+      (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd, (const TP *)gamma, (TDX *)dx,
+      (float *)workspace, rows, (int)C, (const TDX *)dres, pend);
+  return launch_status();
+}
 
 template <typename TDY, typename TX, typename TDX, typename TP>
 int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
               const void *gamma, void *dx, void *dgamma, void *dbeta, void *workspace,
               size_t workspace_bytes, int64_t rows, int64_t C, bool aligned, int x_dtype,
-              int accumulate, const void *dres, hipStream_t s, BwdPhase phase = kBwdWhole) {
+              int accumulate, const void *dres, hipStream_t s, BwdPhase phase = kBwdWhole,
+              PendingSums pending = PendingSums{}) {
   // rows only: the partial rows are the product, the parameter gradients come from a later
-  // cs_layernorm_backward_finalize
+  // cs_layernorm_backward_finalize (or ride in a later call's launch)
   const bool want_dp = phase == kBwdRowsOnly || dgamma != nullptr || dbeta != nullptr;
-  const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
-  if (phase == kBwdRowsOnly && (p.vpl == 0 || std::is_same_v<TX, double>))
+  const BwdPlan plan = aligned ? bwd_plan(rows, C, x_dtype, want_dp, dx != nullptr) : BwdPlan{};
+  if (phase == kBwdRowsOnly && (plan.kind == kBwdNone || std::is_same_v<TX, double>))
     return aligned ? CS_ERR_UNSUPPORTED : CS_ERR_MISALIGNED;
-  // dx + dresidual inside the kernel where it fits (17.5 -> 22 us against 25 us for two
-  // launches at [8192,768] bf16), as a second, in-place launch elsewhere
-  const bool fuse_dres = dres != nullptr && p.vpl != 0 && p.vpl <= kMaxVplWithResidual && is_aligned16(dres);
+  // dx + dresidual inside the kernel where it fits (rows of up to 4 vectors per lane), as a
+  // second, in-place launch elsewhere
+  const bool fuse_dres = dres != nullptr && plan.kind != kBwdNone && plan.vpl <= kMaxVplWithResidual && is_aligned16(dres);
   const void *late_dres = fuse_dres ? nullptr : dres;
   if (!fuse_dres) dres = nullptr;
   if constexpr (!std::is_same_v<TX, double>) {
-    if (p.vpl != 0) {
-      const int blocks =
-          ln_blocks(rows, 1, p.vpl <= 2 ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks, kLnBwdThreads);
-      const int split_blocks = bwd_partial_rows(rows, 8);
-      const int blocks_used = want_dp ? bwd_partial_rows(rows, p.vpl) : blocks;  // partial rows left behind
-      const size_t need = want_dp ? (size_t)blocks_used * 2 * C * sizeof(float) : 0;
+    if (plan.kind != kBwdNone) {
+      const int blocks = plan.blocks;
+      const size_t need = want_dp ? (size_t)blocks * 2 * C * sizeof(float) : 0;
       if (want_dp && (workspace == nullptr || workspace_bytes < need)) return CS_ERR_WORKSPACE;
-      const size_t lds = want_dp ? (size_t)(kLnBwdThreads / kWave) * C * sizeof(float) : 0;
-      const dim3 grid((unsigned)blocks), block(kLnBwdThreads);
+      // the split kernel carries no pending sums: those get their own launch first
+      LnPending pend{nullptr, nullptr, nullptr, 0, 0, 0};
+      if (pending.partial != nullptr && (pending.dgamma != nullptr || pending.dbeta != nullptr)) {
+        if (plan.kind == kBwdSplit) {
+          const int st = launch_finalize<TP>(pending.partial, pending.nparts, pending.dgamma, pending.dbeta, C,
+                                             partial_vn(x_dtype), pending.accumulate, s);
+          if (st != CS_OK) return st;
+        } else {
+          pend = LnPending{(const float *)pending.partial, pending.dgamma, pending.dbeta, (int)pending.nparts,
+                           pending.accumulate, 2 * (int)ceil_div(C, (int64_t)kLnFinCols)};
+        }
+      }
+      size_t lds = want_dp ? plan.fold_lds : 0;
+      const size_t pend_lds = (size_t)kLnFinRows * kLnFinCols * sizeof(float);
+      if (pend.blocks != 0 && lds < pend_lds) lds = pend_lds;
+      const dim3 grid((unsigned)(blocks + pend.blocks)), block(kLnBwdThreads);
+      int st = CS_OK;
 #define CS_LN_BWD(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                       \
   ln_bwd_rows_kernel<TDY, TX, TDX, TP, VPL, WPE, HAS_DX, HAS_DP, HAS_DRES>                  \
       <<<grid, block, lds, s>>>((const TDY *)dy, (const TX *)x, (const float *)mean,        \
                                 (const float *)rstd, (const TP *)gamma, (TDX *)dx,          \
-                                (float *)workspace, rows, (int)C, (const TDX *)dres)
-#define CS_LN_BWD_MASK(VPL, WPE)                \
-  if (dx && want_dp) {                          \
-    CS_LN_BWD(VPL, WPE, true, true, false);     \
+                                (float *)workspace, rows, (int)C, (const TDX *)dres, pend)
+#define CS_LN_K32(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                                          \
+  st = launch_bwd_kernel<TDY, TX, TDX, TP, kLnBwdThreads, 32, VPL, WPE, CS_LN_PAIR_PF, CS_LN_PAIR_KEEP, HAS_DX, \
+                         HAS_DP, HAS_DRES>(dy, x, mean, rstd, gamma, dx, workspace, rows, C, dres, pend, blocks, \
+                                           lds, s)
+#define CS_LN_K64(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                                          \
+  st = launch_bwd_kernel<TDY, TX, TDX, TP, CS_LN_W4_THREADS, 64, VPL, WPE, CS_LN_W4_PF, CS_LN_W4_KEEP, HAS_DX,  \
+                         HAS_DP, HAS_DRES>(dy, x, mean, rstd, gamma, dx, workspace, rows, C, dres, pend, blocks, \
+                                           lds, s)
+#define CS_LN_BWD_MASK(K, VPL, WPE)             \
+  if (dx && want_dp && dres) {                  \
+    K(VPL, WPE, true, true, true);              \
+  } else if (dx && dres) {                      \
+    K(VPL, WPE, true, false, true);             \
+  } else if (dx && want_dp) {                   \
+    K(VPL, WPE, true, true, false);             \
   } else if (dx) {                              \
-    CS_LN_BWD(VPL, WPE, true, false, false);    \
+    K(VPL, WPE, true, false, false);            \
   } else {                                      \
-    CS_LN_BWD(VPL, WPE, false, true, false);    \
+    K(VPL, WPE, false, true, false);            \
   }
-      if (p.vpl == 1 && dres && want_dp) {
-        CS_LN_BWD(1, 4, true, true, true);
-      } else if (p.vpl == 1 && dres) {
-        CS_LN_BWD(1, 4, true, false, true);
-      } else if (p.vpl == 1) {
-        CS_LN_BWD_MASK(1, 4)
-      } else if (p.vpl == 2 && dres && want_dp) {
-        CS_LN_BWD(2, 3, true, true, true);  // four per SIMD would spill
-      } else if (p.vpl == 2 && dres) {
-        CS_LN_BWD(2, 4, true, false, true);
-      } else if (p.vpl == 4 && dres && want_dp) {
-        CS_LN_BWD(4, 2, true, true, true);
-      } else if (p.vpl == 4 && dres) {
-        CS_LN_BWD(4, 2, true, false, true);
-      } else if (p.vpl == 2) {
-        CS_LN_BWD_MASK(2, 4)
-      } else if (p.vpl == 4) {
-        CS_LN_BWD_MASK(4, 2)
-      } else if (want_dp) {
-        // 8 vectors per lane: with the dgamma/dbeta accumulators a row no longer fits one wave's
-        // registers (a single-wave kernel spilled ~1 KB per lane), so two waves share each row
-        const size_t split_lds = (size_t)(kLnBwdThreads / kWave / 2) * 4 * kWave * Vec16<TX>::n * sizeof(float);
-        const dim3 sgrid((unsigned)split_blocks);
+      if (plan.kind == kBwdHalf1) {
+        CS_LN_BWD_MASK(CS_LN_K32, 1, 4)
+      } else if (plan.kind == kBwdHalf3) {
+        CS_LN_BWD_MASK(CS_LN_K32, 3, 2)
+      } else if (plan.kind == kBwdWave4) {
+#if CS_LN_W4_NEW == 2
+        CS_LN_BWD_MASK(CS_LN_K64, 4, CS_LN_W4_WPE)
+#else
+        CS_LN_K64(4, CS_LN_W4_WPE, false, true, false);
+#endif
+      } else if (plan.kind == kBwdSplit) {
         if (dx) {
-          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, true, true><<<sgrid, block, split_lds, s>>>(
+          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, true, true><<<dim3((unsigned)blocks), block, lds, s>>>(
               (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd, (const TP *)gamma,
               (TDX *)dx, (float *)workspace, rows, (int)C);
         } else {
-          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, false, true><<<sgrid, block, split_lds, s>>>(
+          ln_bwd_split_rows_kernel<TDY, TX, TDX, TP, 4, false, true><<<dim3((unsigned)blocks), block, lds, s>>>(
               (const TDY *)dy, (const TX *)x, (const float *)mean, (const float *)rstd, (const TP *)gamma,
               (TDX *)dx, (float *)workspace, rows, (int)C);
         }
+      } else if (plan.vpl == 1) {
+        CS_LN_BWD_MASK(CS_LN_BWD, 1, 4)
+      } else if (plan.vpl == 2 && dres && want_dp) {
+        CS_LN_BWD(2, 3, true, true, true);  // four per SIMD would spill
+      } else if (plan.vpl == 2) {
+        CS_LN_BWD_MASK(CS_LN_BWD, 2, 4)
+      } else if (plan.vpl == 4) {
+        CS_LN_BWD_MASK(CS_LN_BWD, 4, 2)
       } else {
         CS_LN_BWD(8, 2, true, false, false);
       }
 #undef CS_LN_BWD_MASK
+#undef CS_LN_K32
+#undef CS_LN_K64
 #undef CS_LN_BWD
-      int st = launch_status();
-      if (st == CS_OK && want_dp && phase == kBwdWhole) {
-        ln_bwd_finalize_kernel<TP><<<dim3((unsigned)ceil_div(C, (int64_t)kLnFinCols), 2), dim3(kLnFinCols, kLnFinRows), 0, s>>>(
-            (const float *)workspace, blocks_used, (TP *)dgamma, (TP *)dbeta, (int)C, (int)Vec16<TX>::n, accumulate);
-        st = launch_status();
-      }
+      if (st == CS_OK) st = launch_status();
+      if (st == CS_OK && want_dp && phase == kBwdWhole)
+        st = launch_finalize<TP>(workspace, blocks, dgamma, dbeta, C, partial_vn(x_dtype), accumulate, s);
       if (st == CS_OK && late_dres) st = launch_add<TDX>(dx, late_dres, dx, rows * C, s);
       return st;
     }
@@ -1097,10 +1508,13 @@ extern "C" int cs_add_layernorm_forward(const void *x, const void *residual, voi
 
 extern "C" size_t cs_layernorm_backward_workspace_bytes(int64_t rows, int64_t C) {
   if (rows <= 0 || C <= 0) return 0;
-  // the fast path's largest grid: the narrow-row cap, or one row per pair of waves per step
-  const int narrow = ln_blocks(rows, 1, kLnBwdMaxBlocksNarrow, kLnBwdThreads);
-  const int split = ln_blocks(rows, 1, kLnBwdMaxBlocks, kLnBwdThreads / 2);
-  return (size_t)(narrow > split ? narrow : split) * 2 * (size_t)C * sizeof(float);
+  // the most partial rows any plan leaves for this many rows, whatever the storage type
+  int most = 0;
+  for (int dt : {CS_F32, CS_F16}) {
+    const BwdPlan b = bwd_plan(rows, C, dt, true);
+    if (b.blocks > most) most = b.blocks;
+  }
+  return (size_t)most * 2 * (size_t)C * sizeof(float);
 }
 
 namespace {
@@ -1108,7 +1522,7 @@ int ln_backward(const void *dy, const void *x, const void *mean, const void *rst
                 const void *gamma, const void *dres, void *dx, void *dgamma, void *dbeta,
                 void *workspace, size_t workspace_bytes, int64_t rows, int64_t C, int dy_dtype,
                 int x_dtype, int dx_dtype, int param_dtype, int accumulate, void *stream,
-                BwdPhase phase = kBwdWhole) {
+                BwdPhase phase = kBwdWhole, PendingSums pending = PendingSums{}) {
   if (rows < 0 || C <= 0) return CS_ERR_INVALID_ARGUMENT;
   if (dtype_size(x_dtype) == 0 || dtype_size(dy_dtype) == 0 || dtype_size(dx_dtype) == 0 ||
       dtype_size(param_dtype) == 0)
@@ -1139,7 +1553,8 @@ int ln_backward(const void *dy, const void *x, const void *mean, const void *rst
   hipStream_t s = as_stream(stream);
 #define CS_CALL(TDY, TX, TDX, TP)                                                              \
   return bwd_typed<TDY, TX, TDX, TP>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, workspace,   \
-                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, dres, s, phase)
+                                     workspace_bytes, rows, C, aligned, x_dtype, accumulate, dres, s, phase, \
+                                     pending)
   const bool dy_wide = dy_dtype != x_dtype, dx_wide = dx_dtype != x_dtype,
              p_wide = param_dtype != x_dtype;
   switch (x_dtype) {
@@ -1186,8 +1601,7 @@ extern "C" int cs_layernorm_backward_add(const void *dy, const void *x, const vo
 
 extern "C" int64_t cs_layernorm_backward_partial_rows(int64_t rows, int64_t C, int x_dtype) {
   if (rows <= 0 || C <= 0 || dtype_size(x_dtype) == 0) return 0;
-  const FastPlan p = fast_plan(C, x_dtype);
-  return p.vpl == 0 ? 0 : bwd_partial_rows(rows, p.vpl);
+  return bwd_plan(rows, C, x_dtype, true).blocks;
 }
 
 extern "C" int cs_layernorm_backward_rows(const void *dy, const void *x, const void *mean,
@@ -1210,24 +1624,48 @@ extern "C" int cs_layernorm_backward_finalize(const void *partials, int64_t part
   if (dtype_size(x_dtype) == 0 || dtype_size(param_dtype) == 0 || x_dtype == CS_F64 ||
       !wide_ok(x_dtype, param_dtype))
     return CS_ERR_UNSUPPORTED;
-  const int vn = 16 / (int)dtype_size(x_dtype);
-  if (C % vn != 0 || partial_rows > (kLnBwdMaxBlocksNarrow > kLnBwdMaxBlocks ? kLnBwdMaxBlocksNarrow : kLnBwdMaxBlocks))
-    return CS_ERR_INVALID_ARGUMENT;
+  if (C % (16 / (int)dtype_size(x_dtype)) != 0 || partial_rows > kLnMaxPartialRows) return CS_ERR_INVALID_ARGUMENT;
+  const int vn = partial_vn(x_dtype);
   if (!dgamma && !dbeta) return CS_OK;
   if (!is_aligned16(partials) || (dgamma && !aligned_to(dgamma, dtype_size(param_dtype))) ||
       (dbeta && !aligned_to(dbeta, dtype_size(param_dtype))))
     return CS_ERR_MISALIGNED;
   hipStream_t s = as_stream(stream);
-  const dim3 grid((unsigned)ceil_div(C, (int64_t)kLnFinCols), 2), block(kLnFinCols, kLnFinRows);
-#define CS_FIN(TP)                                                                              \
-  ln_bwd_finalize_kernel<TP><<<grid, block, 0, s>>>((const float *)partials, (int)partial_rows, \
-                                                    (TP *)dgamma, (TP *)dbeta, (int)C, vn, accumulate)
   switch (param_dtype) {
-    case CS_F32: CS_FIN(float); break;
-    case CS_F16: CS_FIN(f16_t); break;
-    case CS_BF16: CS_FIN(bf16_t); break;
-    default: return CS_ERR_UNSUPPORTED;
+    case CS_F32: return launch_finalize<float>(partials, partial_rows, dgamma, dbeta, C, vn, accumulate, s);
+    case CS_F16: return launch_finalize<f16_t>(partials, partial_rows, dgamma, dbeta, C, vn, accumulate, s);
+    case CS_BF16: return launch_finalize<bf16_t>(partials, partial_rows, dgamma, dbeta, C, vn, accumulate, s);
   }
-#undef CS_FIN
-  return launch_status();
+  return CS_ERR_UNSUPPORTED;
+}
+
+extern "C" int cs_layernorm_backward_rows_pending(const void *dy, const void *x, const void *mean,
+                                                  const void *rstd, const void *gamma,
+                                                  const void *dresidual, void *dx, void *partials,
+                                                  size_t partials_bytes, const void *pending_partials,
+                                                  int64_t pending_partial_rows, void *pending_dgamma,
+                                                  void *pending_dbeta, int pending_accumulate,
+                                                  int64_t rows, int64_t C, int dy_dtype, int x_dtype,
+                                                  int dx_dtype, int param_dtype, void *stream) {
+  if (rows <= 0 || C <= 0 || !partials || !gamma) return CS_ERR_INVALID_ARGUMENT;
+  if (dresidual && !dx) return CS_ERR_INVALID_ARGUMENT;
+  PendingSums pending;
+  if (pending_partials != nullptr) {
+    if (pending_partial_rows <= 0 || pending_partial_rows > kLnMaxPartialRows) return CS_ERR_INVALID_ARGUMENT;
+    // the sums are read while this call's partial rows are written: they cannot share memory
+    const char *a = (const char *)pending_partials, *b = (const char *)partials;
+    const size_t pend_bytes = (size_t)pending_partial_rows * 2 * (size_t)C * sizeof(float);
+    if (a < b + partials_bytes && b < a + pend_bytes) return CS_ERR_INVALID_ARGUMENT;
+    if (!is_aligned16(pending_partials) || (pending_dgamma && !aligned_to(pending_dgamma, dtype_size(param_dtype))) ||
+        (pending_dbeta && !aligned_to(pending_dbeta, dtype_size(param_dtype))))
+      return CS_ERR_MISALIGNED;
+    pending.partial = pending_partials;
+    pending.nparts = pending_partial_rows;
+    pending.dgamma = pending_dgamma;
+    pending.dbeta = pending_dbeta;
+    pending.accumulate = pending_accumulate;
+  }
+  return ln_backward(dy, x, mean, rstd, gamma, dresidual, dx, nullptr, nullptr, partials,
+                     partials_bytes, rows, C, dy_dtype, x_dtype, dx_dtype, param_dtype, 0, stream,
+                     kBwdRowsOnly, pending);
 }

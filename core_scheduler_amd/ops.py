@@ -349,6 +349,69 @@ def layernorm_backward_finalize(partials, x_dtype, param_dtype, *, need_dgamma=T
     return dgamma, dbeta
 
 
+class LayerNormBackwardChain:
+    """LayerNorm backward calls run one after another on one stream, as a training step runs them
+    (one per norm): each call's launch also adds up the partial rows the PREVIOUS call left, so
+    only the last norm of the chain needs a launch for its column sums (`flush`).
+
+    `backward` returns (dx, dgamma, dbeta) at once; dgamma / dbeta hold their values once the next
+    `backward` of the chain, or `flush`, has run.  The bits are those of `layernorm_backward`.
+    Shapes without partial rows (see `layernorm_backward_rows`) go through `layernorm_backward`.
+    """
+
+    def __init__(self):
+        self._pending = None  # (partials, dgamma, dbeta, accumulate, C, x dtype, parameter dtype)
+
+    def backward(self, dy, x, mean, rstd, gamma, *, dresidual=None, dgamma=None, dbeta=None, dx_dtype=None):
+        dev = _dev(dy, x, mean, rstd, gamma, dgamma, dbeta, dresidual)
+        C = x.shape[-1]
+        rows = x.numel() // C
+        if dresidual is not None and (dresidual.shape != x.shape or dresidual.dtype != (dx_dtype or x.dtype)):
+            raise ValueError("dresidual must match dx")
+        accumulate = dgamma is not None or dbeta is not None
+        if accumulate and (dgamma is None or dbeta is None):
+            raise ValueError("accumulating needs both parameter gradients passed in")
+        for g in (dgamma, dbeta):
+            if g is not None and (g.dtype != gamma.dtype or g.numel() != C):
+                raise ValueError("dgamma / dbeta must be [C] of the parameter dtype")
+        lib = _capi.load()
+        n = lib.cs_layernorm_backward_partial_rows(rows, C, _dt(x))
+        if n == 0:
+            self.flush()
+            return layernorm_backward(dy, x, mean, rstd, gamma, dgamma=dgamma, dbeta=dbeta, dx_dtype=dx_dtype,
+                                      dresidual=dresidual)
+        pend = self._pending
+        if pend is not None and (pend[4], pend[5], pend[6]) != (C, x.dtype, gamma.dtype):
+            self.flush()  # another width or type: its sums cannot ride in this launch
+            pend = None
+        dx = torch.empty(x.shape, dtype=dx_dtype or x.dtype, device=dev)
+        if dgamma is None:
+            dgamma = torch.empty(C, dtype=gamma.dtype, device=dev)
+            dbeta = torch.empty(C, dtype=gamma.dtype, device=dev)
+        partials = torch.empty((n, 2, C), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            code = lib.cs_layernorm_backward_rows_pending(
+                _ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma), _ptr(dresidual), _ptr(dx), _ptr(partials),
+                partials.numel() * 4, _ptr(pend[0]) if pend else None, pend[0].shape[0] if pend else 0,
+                _ptr(pend[1]) if pend else None, _ptr(pend[2]) if pend else None, int(pend[3]) if pend else 0,
+                rows, C, _dt(dy), _dt(x), _dt(dx), _dt(gamma), _stream(dev))
+        _capi.check("cs_layernorm_backward_rows_pending", code)
+        self._pending = (partials, dgamma, dbeta, accumulate, C, x.dtype, gamma.dtype)
+        return dx, dgamma, dbeta
+
+    def flush(self):
+        """Column sums of the last call of the chain, as a launch of their own."""
+        pend, self._pending = self._pending, None
+        if pend is None:
+            return
+        partials, dgamma, dbeta, accumulate, C, x_dtype, p_dtype = pend
+        with torch.cuda.device(partials.device):
+            code = _capi.load().cs_layernorm_backward_finalize(_ptr(partials), partials.shape[0], _ptr(dgamma),
+                                                               _ptr(dbeta), C, _DTYPES[x_dtype], _DTYPES[p_dtype],
+                                                               int(accumulate), _stream(partials.device))
+        _capi.check("cs_layernorm_backward_finalize", code)
+
+
 # -------------------------------------------------------------- Embedding
 def embedding_forward(weight, indices):
     """out[..., :] = weight[indices[...], :] (cs::compute::Embedding::forward)."""

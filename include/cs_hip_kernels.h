@@ -274,6 +274,28 @@ int cs_layernorm_backward_finalize(const void *partials, int64_t partial_rows,
                                    int x_dtype, int param_dtype, int accumulate,
                                    void *stream);
 
+/* cs_layernorm_backward_rows that also does an EARLIER call's
+ * cs_layernorm_backward_finalize inside its own launch: a few workgroups ahead
+ * of the row work add `pending_partials` (what that earlier rows call left,
+ * pending_partial_rows rows of the same C, x_dtype and param_dtype) into
+ * pending_dgamma / pending_dbeta and leave.  A training step runs one
+ * LayerNorm backward after another (src/compute/layer_norm.cpp:228-233, once
+ * per norm, 25 times for GPT-2-small), and the reference already lets the
+ * parameter gradients lag the input gradient (its parameter task runs on the
+ * assist stream, :302,356): each call carries the previous norm's sums, and
+ * only the last norm needs a cs_layernorm_backward_finalize launch of its
+ * own.  Results are those of cs_layernorm_backward_finalize, bit for bit.
+ * pending_partials must not overlap partials (CS_ERR_INVALID_ARGUMENT) and
+ * must have been written by work that precedes this call on the stream;
+ * pending_partials == NULL makes this cs_layernorm_backward_rows. */
+int cs_layernorm_backward_rows_pending(
+    const void *dy, const void *x, const void *mean, const void *rstd,
+    const void *gamma, const void *dresidual, void *dx, void *partials,
+    size_t partials_bytes, const void *pending_partials,
+    int64_t pending_partial_rows, void *pending_dgamma, void *pending_dbeta,
+    int pending_accumulate, int64_t rows, int64_t C, int dy_dtype, int x_dtype,
+    int dx_dtype, int param_dtype, void *stream);
+
 /* ------------------------------------------------------------------------
  * Embedding
  * forward replaces torch::embedding, src/compute/embedding.cpp:117-121:

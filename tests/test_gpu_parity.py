@@ -485,6 +485,8 @@ def test_layernorm_masks_and_accumulate(ops, co):
     (2051, 1600, torch.float32, torch.float32, False),
     (3, 768, torch.float32, torch.float32, False),
     (1500, 384, torch.bfloat16, torch.float32, True),     # one vector per lane
+    (1027, 1600, torch.bfloat16, torch.float32, False),   # four vectors per lane: the sums alone run another kernel
+    (2049, 768, torch.float16, torch.float16, False),     # two rows per wave
 ])
 def test_layernorm_backward_as_two_calls(ops, rows, C, x_dtype, p_dtype, wide_dy):
     """Row pass on one stream, sum of the partial rows on another (the reference's main and
@@ -522,6 +524,77 @@ def test_layernorm_backward_as_two_calls(ops, rows, C, x_dtype, p_dtype, wide_dy
     none_dx, partials_p = ops.layernorm_backward_rows(gdy, gx, gm, gr, gg, need_dx=False)
     assert none_dx is None
     assert_bit_exact(ops.layernorm_backward_finalize(partials_p, x_dtype, p_dtype)[1], whole[2], "dbeta without dx")
+
+
+@pytest.mark.parametrize("rows,C,x_dtype,p_dtype", [
+    (8192, 768, torch.bfloat16, torch.float32),    # benchmark shape: two rows per wave, three vectors per lane
+    (1001, 384, torch.float32, torch.float32),     # the same plan at fp32, odd row count
+    (333, 256, torch.bfloat16, torch.bfloat16),    # two rows per wave, one vector per lane
+    (515, 1600, torch.bfloat16, torch.float32),    # a wave per row, four vectors per lane
+    (64, 1024, torch.float16, torch.float32),      # two vectors per lane
+    (77, 4096, torch.bfloat16, torch.float32),     # two waves per row: pending sums get a launch of their own
+])
+def test_layernorm_backward_chain(ops, rows, C, x_dtype, p_dtype):
+    """Calls whose column sums ride in the next call's launch (cs_layernorm_backward_rows_pending):
+    the bits of cs_layernorm_backward for every call of the chain, with a residual gradient, with
+    accumulation into existing gradients, and across a change of width."""
+    gamma = dev(randn(C, 181, std=0.02, mean=1.0, dtype=p_dtype))
+    calls = []
+    for i in range(4):
+        x = randn((rows, C), 190 + 10 * i, dtype=x_dtype)
+        mean = x.float().mean(-1)
+        rstd = 1.0 / torch.sqrt(x.float().var(-1, unbiased=False) + 1e-5)
+        calls.append(dict(x=dev(x), dy=dev(randn((rows, C), 191 + 10 * i, dtype=x_dtype)), mean=dev(mean), rstd=dev(rstd),
+                          res=dev(randn((rows, C), 192 + 10 * i, dtype=x_dtype)) if i % 2 else None,
+                          acc=(randn(C, 193 + 10 * i, dtype=p_dtype), randn(C, 194 + 10 * i, dtype=p_dtype)) if i == 2 else None))
+    want = []
+    for c in calls:
+        acc = (dev(c["acc"][0]), dev(c["acc"][1])) if c["acc"] else (None, None)
+        want.append(ops.layernorm_backward(c["dy"], c["x"], c["mean"], c["rstd"], gamma, dresidual=c["res"],
+                                           dgamma=acc[0], dbeta=acc[1]))
+    chain = ops.LayerNormBackwardChain()
+    got = []
+    for i, c in enumerate(calls):
+        acc = (dev(c["acc"][0]), dev(c["acc"][1])) if c["acc"] else (None, None)
+        got.append(chain.backward(c["dy"], c["x"], c["mean"], c["rstd"], gamma, dresidual=c["res"],
+                                  dgamma=acc[0], dbeta=acc[1]))
+        if i == 1:
+            # another width in between: the pending sums of call 1 are flushed by the chain itself
+            C2 = 512
+            x2 = dev(randn((40, C2), 300, dtype=x_dtype))
+            m2, r2 = dev(randn(40, 301)), dev(randn(40, 302).abs() + 0.5)
+            g2 = dev(randn(C2, 303, dtype=p_dtype))
+            other = chain.backward(x2, x2, m2, r2, g2)
+            other_want = ops.layernorm_backward(x2, x2, m2, r2, g2)
+    chain.flush()
+    chain.flush()  # nothing pending: no launch, no error
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert_bit_exact(g[0], w[0], f"dx of call {i}")
+        assert_bit_exact(g[1], w[1], f"dgamma of call {i}")
+        assert_bit_exact(g[2], w[2], f"dbeta of call {i}")
+    for a, b, name in zip(other, other_want, ("dx", "dgamma", "dbeta")):
+        assert_bit_exact(a, b, f"{name} of the call of another width")
+
+
+def test_layernorm_backward_pending_rejects_shared_buffers(ops):
+    """The pending partial rows are read while this call's are written: one buffer for both is refused."""
+    import ctypes
+
+    from core_scheduler_amd import _capi
+    lib = _capi.load()
+    rows, C = 64, 768
+    x = dev(randn((rows, C), 310, dtype=torch.bfloat16))
+    m, r, g = dev(randn(rows, 311)), dev(randn(rows, 312).abs() + 0.5), dev(randn(C, 313))
+    n = lib.cs_layernorm_backward_partial_rows(rows, C, _capi.BF16)
+    partials = torch.empty((n, 2, C), dtype=torch.float32, device="cuda:0")
+    dg = torch.empty(C, device="cuda:0")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    dx = torch.empty_like(x)
+    code = lib.cs_layernorm_backward_rows_pending(P(x), P(x), P(m), P(r), P(g), None, P(dx), P(partials), partials.numel() * 4,
+                                                  P(partials), n, P(dg), P(dg), 0, rows, C, _capi.BF16, _capi.BF16,
+                                                  _capi.BF16, _capi.F32, st)
+    assert code == _capi.ERR_INVALID_ARGUMENT
 
 
 def test_layernorm_backward_shapes_without_two_call_form(ops):
