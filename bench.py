@@ -373,6 +373,18 @@ def per_op_table(args, torch, ops):
         add("layernorm_bwd_then_add", f"{tag} [{rows},{C}] bf16, call + torch.add", bwd_bytes + rows * C * 2, mk_res,
             lambda s: torch.add(ops.layernorm_backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma)[0], s["res"]))
 
+        # one call after another, as the norms of a training step: each call's launch also adds up
+        # the partial rows of the call before it (cs_layernorm_backward_rows_pending), so no call
+        # has a launch of its own for the column sums
+        chain = ops.LayerNormBackwardChain()
+        add("layernorm_bwd_chained", f"{tag} [{rows},{C}] bf16, column sums in the next call's launch", bwd_bytes, mk,
+            lambda s: chain.backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma))
+        chain.flush()
+        add("layernorm_bwd_add_chained", f"{tag} [{rows},{C}] bf16, column sums in the next call's launch",
+            bwd_bytes + rows * C * 2, mk_res,
+            lambda s: chain.backward(s["dy"], s["x"], s["mean"], s["rstd"], gamma, dresidual=s["res"]))
+        chain.flush()
+
     # ---- configuration 3: GeLU [8192,3072] bf16, tanh (benchmark) and erf (the reference's form)
     n = 8192 * 3072
     for mode in ("tanh", "none"):
@@ -562,6 +574,7 @@ def per_op_table(args, torch, ops):
                                    [grad[offs[i]:offs[i + 1]] for i in range(len(sizes))],
                                    lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
         keep = {}
+        ln_chain = ops.LayerNormBackwardChain()
 
         def path_step(i):
             k = []
@@ -575,8 +588,9 @@ def per_op_table(args, torch, ops):
             for j in range(L):
                 k.append(ops.gelu_backward(dhs[j], hs[j], "tanh"))
             for j in range(1, n_ln):
-                k.append(ops.layernorm_backward(dys[j], xs[j], mean, rstd, gamma, dresidual=res[j]))
-            k.append(ops.layernorm_backward(dys[0], xs[0], mean, rstd, gamma))
+                k.append(ln_chain.backward(dys[j], xs[j], mean, rstd, gamma, dresidual=res[j]))
+            k.append(ln_chain.backward(dys[0], xs[0], mean, rstd, gamma))
+            ln_chain.flush()  # the first norm's column sums: the one launch of that kind in the step
             k.append(ops.embedding_backward_fused(dout, ids, V))
             opt.step()
             keep[i % 2] = k  # outputs stay alive for a step, as activations and gradients do
@@ -590,7 +604,7 @@ def per_op_table(args, torch, ops):
                   + ln_b + (n_ln - 1) * (ln_b + rows * C * 2)                         # LayerNorm backward
                   + rows * C * 2 + V * C * 2 + T * C * 2                              # embedding backward
                   + 28 * total)                                                       # AdamW
-        launches = 1 + n_ln + L + 3 + L + 2 * n_ln + 3 + 1
+        launches = 1 + n_ln + L + 3 + L + n_ln + 1 + 3 + 1
         path_step(0)
         med, _ = event_ms(path_step, 5, torch)
         out.append({"op": "gpt2_small_step_path", "config": f"B{B} T{T} C{C} {L} blocks V{V}: {launches} launches of the path, "
@@ -756,8 +770,9 @@ def compact_per_op(table):
     cold fraction of the HBM peak.  Everything else a row carries is in the full table."""
     out = []
     for rec in table:
-        cfg = rec["config"].split(",")[0].split(":")[0]
-        out.append({"op": rec["op"], "cfg": cfg[:40], "ms": rec["ms_cold"], "frac": rec["frac_cold"]})
+        parts = rec["config"].split(":")[0].split(", ")
+        cfg = ", ".join(parts[:2]) if rec["op"] == "fused_classifier_call" else parts[0]
+        out.append({"op": rec["op"], "cfg": cfg[:44], "ms": rec["ms_cold"], "frac": rec["frac_cold"]})
     return out
 
 

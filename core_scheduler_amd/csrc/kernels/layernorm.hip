@@ -99,6 +99,23 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
   return to_acc(r.v[i / Vec16<T>::n].e[i % Vec16<T>::n]);
 }
 
+constexpr int kHalf = kWave / 2;
+
+// Sum over the LPR lanes that share a row (all 64, or each half of the wave on its own).
+template <int LPR>
+__device__ __forceinline__ float row_lanes_sum(float v, bool upper) {
+  v += dpp_f32<kDppQuadXor1>(v);
+  v += dpp_f32<kDppQuadXor2>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppRowMirror>(v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  if constexpr (LPR == kWave) return (r0 + r1) + (r2 + r3);
+  return upper ? r2 + r3 : r0 + r1;
+}
+
 // forward launch shape (rows a wave normalises per step, next step's rows prefetched or not)
 #ifndef CS_LN_FWD_ROWS_VPL1
 #define CS_LN_FWD_ROWS_VPL1 4
@@ -121,7 +138,26 @@ __device__ __forceinline__ float raw_get(const Raw<T, N> &r, int i) {
 #ifndef CS_LN_ADD_ROWS_VPL4
 #define CS_LN_ADD_ROWS_VPL4 2
 #endif
-constexpr int kLnThreads = 256;  // 4 waves
+// two rows per wave (rows of up to 32, and of 65-96, vectors): row pairs a wave normalises per step
+#ifndef CS_LN_FWD_HALF
+#define CS_LN_FWD_HALF 1
+#endif
+#ifndef CS_LN_FWD_ROWS_H1
+#define CS_LN_FWD_ROWS_H1 4
+#endif
+#ifndef CS_LN_FWD_ROWS_H3
+#define CS_LN_FWD_ROWS_H3 2
+#endif
+#ifndef CS_LN_ADD_ROWS_H1
+#define CS_LN_ADD_ROWS_H1 4
+#endif
+#ifndef CS_LN_ADD_ROWS_H3
+#define CS_LN_ADD_ROWS_H3 2
+#endif
+#ifndef CS_LN_THREADS
+#define CS_LN_THREADS 256
+#endif
+constexpr int kLnThreads = CS_LN_THREADS;  // 4 waves
 // backward launch shape; the defaults are the measured best, the macros exist for tuning runs
 #ifndef CS_LN_BWD_THREADS
 #define CS_LN_BWD_THREADS 512
@@ -150,16 +186,20 @@ struct RowSet {
   Raw<T, VN> v[R][VPL];
 };
 
-template <typename T, int VN, int VPL, int R>
+template <typename T, int VN, int VPL, int R, int LPR = kWave>
 __device__ __forceinline__ void load_rows(RowSet<T, VN, VPL, R> &dst, const T *__restrict__ src,
                                           int64_t row0, int64_t rows, int C, int nvec, int lane) {
+  // LPR lanes per row: with 32, the wave's halves hold rows row0 + 2r and row0 + 2r + 1
+  constexpr int RPW = kWave / LPR;
+  const int sub = lane / LPR, hl = lane % LPR;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      const int idx = lane + kWave * j;
-      if (idx < nvec && row0 + r < rows) {
-        dst.v[r][j] = load_raw<T, VN>(src + (row0 + r) * C + (int64_t)idx * VN);
+      const int idx = hl + LPR * j;
+      const int64_t row = row0 + r * RPW + sub;
+      if (idx < nvec && row < rows) {
+        dst.v[r][j] = load_raw<T, VN>(src + row * C + (int64_t)idx * VN);
       } else {
         dst.v[r][j] = zero_raw<T, VN>();
       }
@@ -200,28 +240,31 @@ __device__ __forceinline__ void zero_past_row(RowSet<T, VN, VPL, 1> &r, int nvec
 // HAS_RES: the rows that are normalised are x + residual, rounded to x's type (the sum is also
 // written to sum_out, which may be x or residual itself): the residual add in front of the
 // LayerNorm of a transformer block without a [rows, C] round trip between two launches.
-template <typename TX, typename TY, typename TP, int VPL, int R, bool PF, bool HAS_RES>
+template <typename TX, typename TY, typename TP, int VPL, int R, bool PF, bool HAS_RES, int LPR = kWave>
 __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
     const TX *x /* sum_out may be x: not restrict */, const TP *__restrict__ gamma, const TP *__restrict__ beta,
     TY *__restrict__ y, float *__restrict__ mean, float *__restrict__ rstd, int64_t rows, int C,
     float eps, const TX *res, TX *sum_out) {
   constexpr int VN = Vec16<TX>::n;
+  constexpr int RPW = kWave / LPR;  // rows side by side in a wave: R * RPW rows per wave and step
   const int lane = threadIdx.x & (kWave - 1);
+  const int sub = lane / LPR, hl = lane % LPR;
+  const bool upper = sub != 0;
   const int64_t gw = (int64_t)blockIdx.x * (kLnThreads / kWave) + (threadIdx.x >> 6);
-  const int64_t step = (int64_t)gridDim.x * (kLnThreads / kWave) * R;
+  const int64_t step = (int64_t)gridDim.x * (kLnThreads / kWave) * R * RPW;
   const int nvec = C / VN;
-  int64_t row0 = gw * R;
+  int64_t row0 = gw * R * RPW;
   if (row0 >= rows) return;  // wave-uniform
 
   RowSet<TX, VN, VPL, R> cur, rcur;
   if constexpr (PF) {
-    load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
-    if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rcur, res, row0, rows, C, nvec, lane);
+    load_rows<TX, VN, VPL, R, LPR>(cur, x, row0, rows, C, nvec, lane);
+    if constexpr (HAS_RES) load_rows<TX, VN, VPL, R, LPR>(rcur, res, row0, rows, C, nvec, lane);
   }
   float g[VPL][VN], b[VPL][VN];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
-    const int idx = lane + kWave * j;
+    const int idx = hl + LPR * j;
 #pragma unroll
     for (int k = 0; k < VN; ++k) {
       g[j][k] = 0.f;
@@ -237,12 +280,12 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
     RowSet<TX, VN, VPL, R> nxt, rnxt;
     if constexpr (PF) {
       if (row0 + step < rows) {
-        load_rows<TX, VN, VPL, R>(nxt, x, row0 + step, rows, C, nvec, lane);
-        if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rnxt, res, row0 + step, rows, C, nvec, lane);
+        load_rows<TX, VN, VPL, R, LPR>(nxt, x, row0 + step, rows, C, nvec, lane);
+        if constexpr (HAS_RES) load_rows<TX, VN, VPL, R, LPR>(rnxt, res, row0 + step, rows, C, nvec, lane);
       }
     } else {
-      load_rows<TX, VN, VPL, R>(cur, x, row0, rows, C, nvec, lane);
-      if constexpr (HAS_RES) load_rows<TX, VN, VPL, R>(rcur, res, row0, rows, C, nvec, lane);
+      load_rows<TX, VN, VPL, R, LPR>(cur, x, row0, rows, C, nvec, lane);
+      if constexpr (HAS_RES) load_rows<TX, VN, VPL, R, LPR>(rcur, res, row0, rows, C, nvec, lane);
     }
     if constexpr (HAS_RES) {
       // cur = x + residual, one fp32 add and one rounding per element, as an add launch would give
@@ -255,8 +298,9 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
           for (int k = 0; k < VN; ++k)
             sum.e[k] = from_acc<TX>(raw_get<TX, VN>(cur.v[r][j], k) + raw_get<TX, VN>(rcur.v[r][j], k));
           cur.v[r][j].v[0] = sum;
-          const int idx = lane + kWave * j;
-          if (idx < nvec && row0 + r < rows) store16_stream(sum_out + (row0 + r) * C + (int64_t)idx * VN, sum);
+          const int idx = hl + LPR * j;
+          const int64_t row = row0 + r * RPW + sub;
+          if (idx < nvec && row < rows) store16_stream(sum_out + row * C + (int64_t)idx * VN, sum);
         }
       }
     }
@@ -272,13 +316,13 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
       mu[r] = s;
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) mu[r] = wave_reduce(mu[r], SumOp{}) * inv_c;
+    for (int r = 0; r < R; ++r) mu[r] = row_lanes_sum<LPR>(mu[r], upper) * inv_c;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float q = 0.f;
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
-        if (lane + kWave * j < nvec) {
+        if (hl + LPR * j < nvec) {
 #pragma unroll
           for (int k = 0; k < VN; ++k) {
             const float d = raw_get<TX, VN>(cur.v[r][j], k) - mu[r];
@@ -289,23 +333,25 @@ __global__ __launch_bounds__(kLnThreads) void ln_fwd_rows_kernel(
       rs[r] = q;
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) rs[r] = 1.0f / sqrtf(wave_reduce(rs[r], SumOp{}) * inv_c + eps);
+    for (int r = 0; r < R; ++r) rs[r] = 1.0f / sqrtf(row_lanes_sum<LPR>(rs[r], upper) * inv_c + eps);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      if (row0 + r >= rows) break;
-      if (lane == 0) {
-        mean[row0 + r] = mu[r];
-        rstd[row0 + r] = rs[r];
+      if (row0 + r * RPW >= rows) break;  // wave-uniform
+      const int64_t row = row0 + r * RPW + sub;
+      const bool row_ok = row < rows;
+      if (hl == 0 && row_ok) {
+        mean[row] = mu[r];
+        rstd[row] = rs[r];
       }
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
-        const int idx = lane + kWave * j;
-        if (idx < nvec) {
+        const int idx = hl + LPR * j;
+        if (idx < nvec && row_ok) {
           float o[VN];
 #pragma unroll
           for (int k = 0; k < VN; ++k)
             o[k] = (raw_get<TX, VN>(cur.v[r][j], k) - mu[r]) * rs[r] * g[j][k] + b[j][k];
-          store_n<TY, VN>(y + (row0 + r) * C + (int64_t)idx * VN, o);
+          store_n<TY, VN>(y + row * C + (int64_t)idx * VN, o);
         }
       }
     }
@@ -525,23 +571,6 @@ __global__ __launch_bounds__(kLnBwdThreads, WPE) void ln_bwd_rows_kernel(
 // vectors per lane and leaves a quarter of them empty), a wave finishes two rows per round trip to
 // memory, and the same number of waves leaves half as many rows behind them.  The two row sums
 // are reduced per half; the column sums of the halves meet in the LDS fold at the end.
-constexpr int kHalf = kWave / 2;
-
-// Sum over the LPR lanes that share a row (all 64, or each half of the wave on its own).
-template <int LPR>
-__device__ __forceinline__ float row_lanes_sum(float v, bool upper) {
-  v += dpp_f32<kDppQuadXor1>(v);
-  v += dpp_f32<kDppQuadXor2>(v);
-  v += dpp_f32<kDppHalfMirror>(v);
-  v += dpp_f32<kDppRowMirror>(v);
-  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
-  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
-  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
-  if constexpr (LPR == kWave) return (r0 + r1) + (r2 + r3);
-  return upper ? r2 + r3 : r0 + r1;
-}
-
 template <typename T, int VN, int VPL>
 struct Strip {
   Raw<T, VN> v[VPL];
@@ -1122,6 +1151,30 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
   const FastPlan p = aligned ? fast_plan(C, x_dtype) : FastPlan{};
   if constexpr (!std::is_same_v<TX, double>) {
     if (p.vpl != 0) {
+      // rows of up to 32 vectors, and of 65 to 96 (C = 768 at 16 bit), go two to a wave: no lane
+      // slot stays empty
+      const int64_t nvec = C / Vec16<TX>::n;
+      const int half_vpl = !CS_LN_FWD_HALF ? 0 : nvec <= kHalf ? 1 : (nvec > kWave && nvec <= 3 * kHalf) ? 3 : 0;
+      if (half_vpl != 0) {
+        const int groups = res ? (half_vpl == 1 ? CS_LN_ADD_ROWS_H1 : CS_LN_ADD_ROWS_H3)
+                               : (half_vpl == 1 ? CS_LN_FWD_ROWS_H1 : CS_LN_FWD_ROWS_H3);
+        const dim3 grid((unsigned)ln_blocks(rows, 2 * groups, kLnFwdMaxBlocks)), block(kLnThreads);
+#define CS_LN_FWD_H(VPL, R, HAS_RES)                                                                 \
+  ln_fwd_rows_kernel<TX, TY, TP, VPL, R, CS_LN_FWD_PF, HAS_RES, kHalf><<<grid, block, 0, s>>>(       \
+      (const TX *)x, (const TP *)gamma, (const TP *)beta, (TY *)y, (float *)mean, (float *)rstd, rows, \
+      (int)C, (float)eps, (const TX *)res, (TX *)sum_out)
+        if (res && half_vpl == 1) {
+          CS_LN_FWD_H(1, CS_LN_ADD_ROWS_H1, true);
+        } else if (res) {
+          CS_LN_FWD_H(3, CS_LN_ADD_ROWS_H3, true);
+        } else if (half_vpl == 1) {
+          CS_LN_FWD_H(1, CS_LN_FWD_ROWS_H1, false);
+        } else {
+          CS_LN_FWD_H(3, CS_LN_FWD_ROWS_H3, false);
+        }
+#undef CS_LN_FWD_H
+        return launch_status();
+      }
       // with the residual stream a wave holds two inputs per row: half the rows per step
       const int r_rows = res ? (p.vpl == 1   ? CS_LN_ADD_ROWS_VPL1
                                 : p.vpl == 2 ? CS_LN_ADD_ROWS_VPL2

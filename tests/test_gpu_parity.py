@@ -336,6 +336,10 @@ def _ln_case(ops, co, rows, C, x_dtype, p_dtype, bias=True, atol_y=2e-6):
     (2049, 50, torch.float32, torch.float32),       # the same with long column sums
     (33, 10000, torch.bfloat16, torch.float32),     # beyond the register plans
     (128, 384, torch.float64, torch.float64),       # test/test_layer_norm.cpp:99-134
+    (301, 256, torch.bfloat16, torch.float32),      # two rows per wave, one vector per lane, odd row count
+    (1001, 128, torch.float32, torch.float32),      # the same from fp32 rows
+    (999, 760, torch.bfloat16, torch.float32),      # two rows per wave, 95 of 96 vector slots used
+    (7, 24, torch.float16, torch.float16),          # three vectors per row
 ])
 def test_layernorm(ops, co, rows, C, x_dtype, p_dtype):
     _ln_case(ops, co, rows, C, x_dtype, p_dtype)
@@ -353,6 +357,8 @@ def test_layernorm(ops, co, rows, C, x_dtype, p_dtype):
     (64, 50, torch.float32, torch.float32),         # general path
     (33, 10000, torch.bfloat16, torch.float32),     # general path
     (128, 384, torch.float64, torch.float64),
+    (301, 256, torch.bfloat16, torch.float32),      # two rows per wave, one vector per lane, odd row count
+    (999, 760, torch.bfloat16, torch.float32),      # two rows per wave, 95 of 96 vector slots used
 ])
 def test_layernorm_with_residual_stream(ops, co, rows, C, x_dtype, p_dtype):
     """x + residual -> LayerNorm, and LayerNorm backward + dresidual, each in one pass
