@@ -411,14 +411,39 @@ def per_op_table(args, torch, ops):
                     return torch.randint(0, V, (B, T), generator=g, device=dev, dtype=torch.int64)
                 return torch.multinomial(ranks / ranks.sum(), B * T, replacement=True, generator=g).reshape(B, T)
 
+            distinct = []
+
             def mk_fwd():
-                return {"wte": randn((V, C), 0.02), "wpe": randn((T, C), 0.02), "ids": mk_ids()}
+                ids_ = mk_ids()
+                distinct.append(int(torch.unique(ids_).numel()))
+                return {"wte": randn((V, C), 0.02), "wpe": randn((T, C), 0.02), "ids": ids_}
 
             def mk_bwd():
                 return {"dout": randn((B, T, C)), "ids": mk_ids()}
 
+            # a table row that several tokens name is read from memory once: the bytes that have to
+            # move count each distinct row once (measured for this row's own id sets), which is what
+            # the fraction of the HBM peak is taken against; `bytes_every_token_row` keeps the figure
+            # that counts one table row per token
+            n_before = len(out)
             add("embedding_fwd", f"{tag} {kind} B{B} T{T} C{C}", fwd_bytes, mk_fwd,
                 lambda s: ops.embedding_forward_add(s["wte"], s["wpe"], s["ids"]))
+            if len(out) > n_before and distinct:
+                rec = out[-1]
+                rows_read = sum(distinct) / len(distinct)
+                nb = int(B * T * 8 + rows_read * C * 2 + T * C * 2 + B * T * C * 2)
+                rec["bytes_every_token_row"] = fwd_bytes
+                rec["distinct_rows_mean"] = round(rows_read, 1)
+                rec["algorithmic_bytes"] = nb
+                for k, ms in (("warm", rec["ms_warm"]), ("cold", rec["ms_cold"])):
+                    rec[f"gbps_{k}"] = round(nb / ms / 1e6, 1)
+                rec["frac_cold"] = round(nb / rec["ms_cold"] / 1e6 / HBM_PEAK_GBPS, 4)
+                ceiling = copy_ms_at(nb)
+                if ceiling:
+                    rec["copy_ms_same_bytes"] = round(ceiling, 5)
+                    rec["frac_of_copy"] = round(ceiling / rec["ms_cold"], 3)
+                log(f"[per-op]   distinct table rows {rows_read:.0f} of {B * T} tokens: {nb} bytes have to move, "
+                    f"{rec['gbps_cold']:.1f} GB/s, {rec['frac_cold']*100:.1f}% of HBM peak")
             add("embedding_bwd", f"{tag} {kind} B{B} T{T} C{C}", bwd_bytes, mk_bwd,
                 lambda s: ops.embedding_backward_fused(s["dout"], s["ids"], V))
 
