@@ -111,6 +111,10 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 4 + [c_size_t] + [c_int64] * 4 + [c_int, c_int, c_int, c_void_p],
     ),
+    "cs_embedding_backward_scaled": (
+        c_int,
+        [c_void_p] * 4 + [c_size_t] + [c_int64] * 4 + [c_int, c_int, c_int, c_void_p],
+    ),
     "cs_embedding_backward_fused": (
         c_int,
         [c_void_p] * 5 + [c_size_t] + [c_int64] * 4 + [c_int, c_int, c_int, c_void_p],

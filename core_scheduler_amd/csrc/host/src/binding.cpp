@@ -165,15 +165,19 @@ PYBIND11_MODULE(_cs_host, m) {
         .def("zero_grad", &Op::State::zero_grad);
     auto sub = m.def_submodule("Embedding");
     sub.def("init", [](const Scheduler &s, int64_t n, int64_t d, std::optional<int64_t> padding_idx,
-                       std::optional<double> max_norm, const std::string &dtype) {
+                       std::optional<double> max_norm, const std::string &dtype, bool scale_grad_by_freq,
+                       bool sparse) {
       auto o = Op::Options{n, d}
                    .device(at::Device(at::kCUDA, device_of(s)))
-                   .dtype(dtype_from(dtype));
+                   .dtype(dtype_from(dtype))
+                   .scale_grad_by_freq(scale_grad_by_freq)
+                   .sparse(sparse);
       if (padding_idx) o = o.padding_idx(*padding_idx);
       if (max_norm) o = o.max_norm(*max_norm);
       return Op::init(s, o);
     }, py::arg("scheduler"), py::arg("num_embeddings"), py::arg("embedding_dim"),
-            py::arg("padding_idx") = py::none(), py::arg("max_norm") = py::none(), py::arg("dtype") = "float32");
+            py::arg("padding_idx") = py::none(), py::arg("max_norm") = py::none(), py::arg("dtype") = "float32",
+            py::arg("scale_grad_by_freq") = false, py::arg("sparse") = false);
     sub.def("forward", &Op::forward);
     sub.def("backward", &Op::backward);
     sub.def("forward_with_positions", &Op::forward_with_positions);

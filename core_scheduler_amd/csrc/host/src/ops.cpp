@@ -280,7 +280,8 @@ void Embedding::backward(const Scheduler &scheduler, const std::shared_ptr<State
          const State::Args &a)
         : Task::Impl{std::move(out), std::move(in), kAssist, kCompute}, args{a} {}
     void operator()() const override {
-      CS_ASSERT_TRUE(!args.scale_grad_by_freq && !args.sparse, "scale_grad_by_freq / sparse are not supported");
+      // `sparse` would return a sparse tensor (at::embedding_backward's other branch): not built
+      CS_ASSERT_TRUE(!args.sparse, "sparse embedding gradients are not supported");
       const at::Tensor dout = T(input()[0]).contiguous();
       const at::Tensor idx = T(input()[1]).contiguous();
       at::Tensor &gw = T(output()[0]);
@@ -293,9 +294,10 @@ void Embedding::backward(const Scheduler &scheduler, const std::shared_ptr<State
                   "Embedding::backward: the existing gradient must be a contiguous [num_embeddings, C] tensor of "
                   "grad_output's dtype");
       at::Tensor ws = workspace(cs_embedding_backward_workspace_bytes(idx.numel(), C, args.num_weights), dout);
-      check(cs_embedding_backward(dout.data_ptr(), idx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws.numel(),
-                                  idx.numel(), C, args.num_weights, args.padding_idx, dtype_of(dout.scalar_type()),
-                                  itype_of(idx.scalar_type()), accumulate ? 1 : 0, current_stream()),
+      const auto kernel = args.scale_grad_by_freq ? cs_embedding_backward_scaled : cs_embedding_backward;
+      check(kernel(dout.data_ptr(), idx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws.numel(), idx.numel(), C,
+                   args.num_weights, args.padding_idx, dtype_of(dout.scalar_type()), itype_of(idx.scalar_type()),
+                   accumulate ? 1 : 0, current_stream()),
             name());
       intermediate().push_back(ws);
     }

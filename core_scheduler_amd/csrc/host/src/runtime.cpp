@@ -45,9 +45,12 @@ struct Event::Impl {
 
  private:
   // Events here order streams of one device and tell the host that work has finished; the data
-  // itself reaches the host through stream-ordered copies.  Without the system-scope fence a
-  // record costs the stream 0.9 us instead of 2.7 us (measured behind a 14 us kernel).
-  at::cuda::CUDAEvent event{hipEventDisableTiming | hipEventDisableSystemFence};
+  // itself reaches the host through stream-ordered copies.  hipEventReleaseToDevice is the
+  // runtime's flag for exactly that: a record releases at device scope, so the stream waits,
+  // queries and host synchronisations that the scheduler builds on these events synchronize
+  // with the recorded work for every reader on this device, without the write-back to system
+  // scope of a default event (which costs the recording stream ~2.7 us here instead of ~0.9 us).
+  at::cuda::CUDAEvent event{hipEventDisableTiming | hipEventReleaseToDevice};
 };
 
 namespace {

@@ -611,7 +611,7 @@ template <typename T>
 __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduce_kernel(
     const T *__restrict__ dout, const uint32_t *__restrict__ sorted_id,
     const uint32_t *__restrict__ sorted_pos, T *__restrict__ dweight, float *__restrict__ partial,
-    int64_t n, int64_t C, int accumulate) {
+    int64_t n, int64_t C, int accumulate, int by_freq) {
   constexpr int VN = Vec16<T>::n;
   constexpr int kChunkCols = kWave * kVpl * VN;
   extern __shared__ float lds[];  // [kRedWaves][2 slots][kChunkCols]
@@ -707,6 +707,8 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
         const bool seg_ends = !(q + 1 >= n_valid && leaves);
         if (seg_begins && seg_ends) {
           T *dst = dweight + (int64_t)id * C;
+          // scale_grad_by_freq: the sum over the id's entries divided by their number
+          const float inv = by_freq ? 1.0f / (float)(q - piece_start + 1) : 1.0f;
 #pragma unroll
           for (int j = 0; j < kVpl; ++j) {
             const int idx = cb + lane + kWave * j;
@@ -715,10 +717,10 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
               if (accumulate) {
                 const Vec16<T> old = load16(dst + (int64_t)idx * VN);
 #pragma unroll
-                for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(to_acc(old.e[k]) + acc[j][k]);
+                for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(to_acc(old.e[k]) + acc[j][k] * inv);
               } else {
 #pragma unroll
-                for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(acc[j][k]);
+                for (int k = 0; k < VN; ++k) o.e[k] = from_acc<T>(acc[j][k] * inv);
               }
               store16_stream(dst + (int64_t)idx * VN, o);
             }
@@ -793,9 +795,10 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
           const int64_t col = ((int64_t)cb + lane + kWave * (v / H)) * VN + 4 * (v % H);
           if (col >= C) continue;  // C is a multiple of VN columns here
           if (whole) {
+            const float inv = by_freq ? 1.0f / (float)(b - a) : 1.0f;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-              float o = t[v][k];
+              float o = t[v][k] * inv;
               if (accumulate) o += to_acc(drow[col + k]);
               drow[col + k] = from_acc<T>(o);
             }
@@ -818,7 +821,7 @@ __global__ __launch_bounds__(kRedThreads, 2048 / kRedThreads) void emb_bwd_reduc
 template <typename T>
 __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
     const uint32_t *__restrict__ sorted_id, const float *__restrict__ partial,
-    T *__restrict__ dweight, int64_t n, int64_t C, int accumulate) {
+    T *__restrict__ dweight, int64_t n, int64_t C, int accumulate, int by_freq) {
   __shared__ int first_other[kFinWaves];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -852,6 +855,17 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
   // its first entry still has the id, otherwise exactly at the end of the window before.
   const bool tail = w_hi * kWindow < n && sorted_id[w_hi * kWindow] == id;
   const int64_t w_end = tail ? w_hi : w_hi - 1;  // the window the segment ends in (> w)
+  // scale_grad_by_freq: the segment's length, from where it begins in window w to where it ends
+  // in window w_end (it fills every window in between)
+  float inv = 1.0f;
+  if (by_freq) {
+    const int64_t qa = w * kWindow + (lane < kWindow ? lane : kWindow - 1);
+    const int64_t qb = w_end * kWindow + (lane < kWindow ? lane : kWindow - 1);
+    const uint64_t in_first = __ballot(lane < kWindow && sorted_id[qa] == id);                        // a suffix of window w
+    const uint64_t in_last = __ballot(lane < kWindow && qb < n && sorted_id[qb < n ? qb : n - 1] == id);  // a prefix of window w_end
+    const int64_t count = __popcll(in_first) + (w_end - w - 1) * kWindow + __popcll(in_last);
+    inv = 1.0f / (float)count;
+  }
   T *dst = dweight + (int64_t)id * C;
   for (int64_t col = tid; col < C; col += kFinThreads) {
     // eight interleaved sums keep eight loads in flight; the order is fixed all the same
@@ -873,7 +887,7 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
       for (int u = 0; u < 7; ++u) t[u] += v[u];  // at most seven windows are left
     }
     t[7] += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
-    float total = ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+    float total = (((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]))) * inv;
     if (accumulate) total += to_acc(dst[col]);
     dst[col] = from_acc<T>(total);
   }
@@ -912,7 +926,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void emb_bwd_rows_general_kernel(
     const T *__restrict__ dout, const uint32_t *__restrict__ sorted_id,
     const uint32_t *__restrict__ sorted_pos, T *__restrict__ dweight, int64_t n, int64_t C,
-    int accumulate) {
+    int accumulate, int by_freq) {
   using U = typename Acc<T>::type;
   const uint32_t row = blockIdx.x;
   // first sorted entry with id >= row (unused tail slots hold kNoId, the maximum)
@@ -927,8 +941,10 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_rows_general_kernel(
   // row drift by ~1e-4 of the terms' scale, so this path, which is not the fast one, adds in double.
   for (int64_t c = threadIdx.x; c < C; c += kThreads) {
     double a = 0;
-    for (int64_t p = lo; p < n && sorted_id[p] == row; ++p)
+    int64_t count = 0;
+    for (int64_t p = lo; p < n && sorted_id[p] == row; ++p, ++count)
       a += (double)to_acc(dout[(int64_t)sorted_pos[p] * C + c]);
+    if (by_freq && count > 0) a /= (double)count;  // scale_grad_by_freq
     if (accumulate) a += (double)to_acc(dweight[(int64_t)row * C + c]);
     dweight[(int64_t)row * C + c] = from_acc<T>((U)a);
   }
@@ -1010,6 +1026,10 @@ int fwd_dispatch(const void *weight, const void *wpe, const void *ids, void *out
   if (idx_dtype != CS_I32 && idx_dtype != CS_I64) return CS_ERR_INVALID_ARGUMENT;
   if (n_rows == 0) return CS_OK;
   if (!weight || !ids || !out || (ADD && !wpe)) return CS_ERR_INVALID_ARGUMENT;
+  // an empty table has no row 0 for the lanes that read it in place of an out-of-range id
+  if (num_weights == 0) return CS_ERR_INVALID_ARGUMENT;
+  // the vector kernel keeps the position-table length in 32 bits
+  if (ADD && T_len > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
   if (!aligned_to(weight, es) || !aligned_to(out, es) || (ADD && !aligned_to(wpe, es)) ||
       !aligned_to(ids, idx_dtype == CS_I64 ? 8 : 4))
     return CS_ERR_MISALIGNED;
@@ -1113,7 +1133,7 @@ int allow_reduce_lds(size_t bytes) {
 template <typename T>
 int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char *ws,
               const BwdLayout &L, int64_t n, int64_t C, int64_t num_weights, int64_t padding_idx,
-              int64_t B, int64_t T_len, int idx_dtype, int accumulate, hipStream_t s) {
+              int64_t B, int64_t T_len, int idx_dtype, int accumulate, int by_freq, hipStream_t s) {
   constexpr int VN = Vec16<T>::n;
   const bool vec_ok = !std::is_same_v<T, double> && C % VN == 0 && is_aligned16(dout) &&
                       is_aligned16(dweight) && (!dwpe || is_aligned16(dwpe));
@@ -1138,7 +1158,7 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
   if (!vec_ok) {
     if (num_weights > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
     emb_bwd_rows_general_kernel<T><<<dim3((unsigned)num_weights), dim3(kThreads), 0, s>>>(
-        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, n, C, accumulate);
+        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, n, C, accumulate, by_freq);
     st = launch_status();
     if (st != CS_OK || !dwpe) return st;
     int64_t blocks = ceil_div(TC, (int64_t)kThreads);
@@ -1156,11 +1176,11 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
     st = allow_reduce_lds<T>(lds);
     if (st != CS_OK) return st;
     emb_bwd_reduce_kernel<T><<<dim3((unsigned)windows), dim3(kRedThreads), lds, s>>>(
-        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, partial, n, C, accumulate);
+        (const T *)dout, sorted_id, sorted_pos, (T *)dweight, partial, n, C, accumulate, by_freq);
     st = launch_status();
     if (st != CS_OK) return st;
     emb_bwd_finish_kernel<T><<<dim3((unsigned)windows), dim3(kFinThreads), 0, s>>>(
-        sorted_id, partial, (T *)dweight, n, C, accumulate);
+        sorted_id, partial, (T *)dweight, n, C, accumulate, by_freq);
     return launch_status();
   }
   return CS_ERR_UNSUPPORTED;
@@ -1169,7 +1189,7 @@ int bwd_typed(const void *dout, const void *ids, void *dweight, void *dwpe, char
 int bwd_dispatch(const void *dout, const void *ids, void *dweight, void *dwpe, void *workspace,
                  size_t workspace_bytes, int64_t n, int64_t C, int64_t num_weights,
                  int64_t padding_idx, int64_t B, int64_t T_len, int dtype, int idx_dtype,
-                 int accumulate, void *stream) {
+                 int accumulate, void *stream, int by_freq = 0) {
   if (n < 0 || C <= 0 || num_weights <= 0) return CS_ERR_INVALID_ARGUMENT;
   const size_t es = dtype_size(dtype);
   if (es == 0) return CS_ERR_UNSUPPORTED;
@@ -1187,16 +1207,16 @@ int bwd_dispatch(const void *dout, const void *ids, void *dweight, void *dwpe, v
   switch (dtype) {
     case CS_F32:
       return bwd_typed<float>(dout, ids, dweight, dwpe, ws, L, n, C, num_weights, padding_idx, B,
-                              T_len, idx_dtype, accumulate, s);
+                              T_len, idx_dtype, accumulate, by_freq, s);
     case CS_F64:
       return bwd_typed<double>(dout, ids, dweight, dwpe, ws, L, n, C, num_weights, padding_idx, B,
-                               T_len, idx_dtype, accumulate, s);
+                               T_len, idx_dtype, accumulate, by_freq, s);
     case CS_F16:
       return bwd_typed<f16_t>(dout, ids, dweight, dwpe, ws, L, n, C, num_weights, padding_idx, B,
-                              T_len, idx_dtype, accumulate, s);
+                              T_len, idx_dtype, accumulate, by_freq, s);
     case CS_BF16:
       return bwd_typed<bf16_t>(dout, ids, dweight, dwpe, ws, L, n, C, num_weights, padding_idx, B,
-                               T_len, idx_dtype, accumulate, s);
+                               T_len, idx_dtype, accumulate, by_freq, s);
   }
   return CS_ERR_UNSUPPORTED;
 }
@@ -1234,6 +1254,14 @@ extern "C" int cs_embedding_backward(const void *dout, const void *indices, void
                                      int dtype, int idx_dtype, int accumulate, void *stream) {
   return bwd_dispatch(dout, indices, dweight, nullptr, workspace, workspace_bytes, n_indices, C,
                       num_weights, padding_idx, 0, 1, dtype, idx_dtype, accumulate, stream);
+}
+
+extern "C" int cs_embedding_backward_scaled(const void *dout, const void *indices, void *dweight,
+                                            void *workspace, size_t workspace_bytes, int64_t n_indices,
+                                            int64_t C, int64_t num_weights, int64_t padding_idx,
+                                            int dtype, int idx_dtype, int accumulate, void *stream) {
+  return bwd_dispatch(dout, indices, dweight, nullptr, workspace, workspace_bytes, n_indices, C,
+                      num_weights, padding_idx, 0, 1, dtype, idx_dtype, accumulate, stream, 1);
 }
 
 extern "C" int cs_embedding_backward_fused(const void *dout, const void *indices, void *dwte,

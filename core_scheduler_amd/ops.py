@@ -446,8 +446,9 @@ def _check_table_gradient(t, rows, C, dtype, name):
         raise ValueError(f"{name} must be a contiguous [{rows}, {C}] tensor of {dtype}, got {tuple(t.shape)} {t.dtype}")
 
 
-def embedding_backward(dout, indices, num_weights, padding_idx=-1, dweight=None):
-    """Dense dweight [num_weights, C]; passing dweight accumulates into it."""
+def embedding_backward(dout, indices, num_weights, padding_idx=-1, dweight=None, scale_grad_by_freq=False):
+    """Dense dweight [num_weights, C]; passing dweight accumulates into it.  `scale_grad_by_freq`
+    divides a row's sum by the number of indices that name it."""
     C = dout.shape[-1]
     n = indices.numel()
     accumulate = dweight is not None
@@ -460,9 +461,9 @@ def embedding_backward(dout, indices, num_weights, padding_idx=-1, dweight=None)
     ws_bytes = lib.cs_embedding_backward_workspace_bytes(n, C, num_weights)
     ws = _workspace(ws_bytes, dev)
     with torch.cuda.device(dev):
-        code = lib.cs_embedding_backward(_ptr(dout), _ptr(indices), _ptr(dweight), _ptr(ws), ws_bytes, n, C,
-                                         num_weights, padding_idx, _dt(dout), _ITYPES[indices.dtype],
-                                         int(accumulate), _stream(dev))
+        call = lib.cs_embedding_backward_scaled if scale_grad_by_freq else lib.cs_embedding_backward
+        code = call(_ptr(dout), _ptr(indices), _ptr(dweight), _ptr(ws), ws_bytes, n, C, num_weights, padding_idx,
+                    _dt(dout), _ITYPES[indices.dtype], int(accumulate), _stream(dev))
     _capi.check("cs_embedding_backward", code)
     return dweight
 

@@ -331,6 +331,19 @@ int cs_embedding_backward(const void *dout, const void *indices,
                           int64_t num_weights, int64_t padding_idx, int dtype,
                           int idx_dtype, int accumulate, void *stream);
 
+/* cs_embedding_backward with the reference's scale_grad_by_freq option
+ * (at::embedding_backward(..., scale_grad_by_freq = true, sparse = false),
+ * src/compute/embedding.cpp:147-157): the gradient of a row is the sum over
+ * the entries that name it divided by their number, then added to what is
+ * there when accumulate != 0.  (The `sparse` option returns a sparse tensor
+ * and has no counterpart here.) */
+int cs_embedding_backward_scaled(const void *dout, const void *indices,
+                                 void *dweight, void *workspace,
+                                 size_t workspace_bytes, int64_t n_indices,
+                                 int64_t C, int64_t num_weights,
+                                 int64_t padding_idx, int dtype, int idx_dtype,
+                                 int accumulate, void *stream);
+
 /* Token and position table gradients of out[b,t,:] = wte[ids[b,t],:] +
  * wpe[t,:] from one dout[B,T,C]: dwte as cs_embedding_backward (no padding
  * index), dwpe[t,:] (+)= sum_b dout[b,t,:] in ascending b.  Replaces

@@ -41,9 +41,9 @@ def embedding_forward(weight, indices, padding_idx=-1):
     return aten.embedding(weight, indices.view(-1, indices.size(-1)), padding_idx, False, False)
 
 
-def embedding_backward(grad_output, indices, num_weights, padding_idx=-1):
-    """src/compute/embedding.cpp:147-157 (the `=` branch)"""
-    return aten.embedding_backward(grad_output, indices, num_weights, padding_idx, False, False)
+def embedding_backward(grad_output, indices, num_weights, padding_idx=-1, scale_grad_by_freq=False):
+    """src/compute/embedding.cpp:147-157 (the `=` branch); `sparse` stays false"""
+    return aten.embedding_backward(grad_output, indices, num_weights, padding_idx, scale_grad_by_freq, False)
 
 
 def token_position_forward(wte, wpe, ids):

@@ -149,14 +149,14 @@ def embedding_forward_add(wte, wpe, ids):
     return out.to(wte.dtype)
 
 
-def embedding_backward(dout, ids, num_weights, padding_idx=-1, dweight=None):
+def embedding_backward(dout, ids, num_weights, padding_idx=-1, dweight=None, scale_grad_by_freq=False):
     dw, sfx = _wide(dout)
     C = dout.shape[-1]
     idx = _ids(ids)
     acc = dweight is not None
     g = _wide(dweight)[0] if acc else torch.empty(num_weights, C, dtype=dw.dtype)
     _call("oracle_embedding_backward", sfx, _p(dw), _p(idx), _p(g), I64(idx.numel()), I64(C), I64(num_weights),
-          I64(padding_idx), INT(int(acc)))
+          I64(padding_idx), INT(int(acc)), INT(int(scale_grad_by_freq)))
     return g.to(dout.dtype)
 
 

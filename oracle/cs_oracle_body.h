@@ -195,20 +195,27 @@ void FN(oracle_embedding_forward_add)(const REAL *wte, const REAL *wpe, const in
     }
 }
 
-/* ---- Embedding backward: at::embedding_backward (dense) and the += of an
- * existing gradient, src/compute/embedding.cpp:147-157.  Rows equal to
- * padding_idx get nothing; padding_idx < 0 means none. */
+/* ---- Embedding backward: at::embedding_backward (dense, with and without
+ * scale_grad_by_freq) and the += of an existing gradient,
+ * src/compute/embedding.cpp:147-157.  Rows equal to padding_idx get nothing;
+ * padding_idx < 0 means none. */
 void FN(oracle_embedding_backward)(const REAL *dout, const int64_t *ids, REAL *dweight,
                                    int64_t n, int64_t C, int64_t V, int64_t padding_idx,
-                                   int accumulate) {
+                                   int accumulate, int scale_grad_by_freq) {
   double *acc = (double *)calloc((size_t)(V * C), sizeof(double));
+  int64_t *count = (int64_t *)calloc((size_t)V, sizeof(int64_t));
   for (int64_t i = 0; i < n; ++i) {
     const int64_t id = ids[i];
     if (id < 0 || id >= V || id == padding_idx) continue;
+    count[id] += 1;
     for (int64_t c = 0; c < C; ++c) acc[id * C + c] += dout[i * C + c];
   }
-  for (int64_t k = 0; k < V * C; ++k)
-    dweight[k] = (REAL)(acc[k] + (accumulate ? (double)dweight[k] : 0.0));
+  /* scale_grad_by_freq: every contribution to row k weighs 1 / (entries naming k) */
+  for (int64_t k = 0; k < V * C; ++k) {
+    const double scale = (scale_grad_by_freq && count[k / C] > 0) ? 1.0 / (double)count[k / C] : 1.0;
+    dweight[k] = (REAL)(acc[k] * scale + (accumulate ? (double)dweight[k] : 0.0));
+  }
+  free(count);
   free(acc);
 }
 

@@ -69,6 +69,16 @@ def test_argument_checks_reject_before_launch():
     assert lib.cs_embedding_forward(p, p, p, 4, 8, 10, _capi.F32, 5, None) == _capi.ERR_INVALID_ARGUMENT
     assert lib.cs_embedding_backward(p, p, p, None, 0, 4, 8, 10, -1, _capi.F32, _capi.I64, 0,
                                      None) == _capi.ERR_WORKSPACE
+    # an empty table cannot be gathered from; a position table longer than 2^31 - 1 rows is refused
+    assert lib.cs_embedding_forward(p, p, p, 4, 8, 0, _capi.F32, _capi.I64, None) == _capi.ERR_INVALID_ARGUMENT
+    assert lib.cs_embedding_forward(p, p, p, 0, 8, 0, _capi.F32, _capi.I64, None) == _capi.OK  # nothing to gather
+    assert lib.cs_embedding_forward_add(p, p, p, p, 1, 1 << 31, 8, 10, _capi.F32, _capi.I64, None) == _capi.ERR_TOO_LARGE
+    # the pending partial rows of cs_layernorm_backward_rows_pending may not be this call's own
+    assert lib.cs_layernorm_backward_rows_pending(p, p, p, p, p, None, p, p, 1 << 20, p, 4, p, p, 0, 64, 768, _capi.BF16,
+                                                  _capi.BF16, _capi.BF16, _capi.F32, None) == _capi.ERR_INVALID_ARGUMENT
+    assert lib.cs_layernorm_backward_rows_pending(p, p, p, p, p, None, p, p, 1 << 20, ctypes.c_void_p(1 << 30), 100000, p, p,
+                                                  0, 64, 768, _capi.BF16, _capi.BF16, _capi.BF16, _capi.F32,
+                                                  None) == _capi.ERR_INVALID_ARGUMENT  # more rows than any plan leaves
     assert lib.cs_fused_classifier(p, p, p, p, p, p, p, 1 << 20, 4, 100, 50, -100, 1, 1.0, _capi.BF16, _capi.BF16,
                                    None) == _capi.ERR_INVALID_ARGUMENT  # stride < V
     assert lib.cs_fused_classifier(p, p, p, p, p, p, None, 0, 4, 100, 128, -100, 1, 1.0, _capi.BF16, _capi.BF16,

@@ -682,6 +682,38 @@ def test_embedding_backward_padding_accumulate_and_bad_ids(ops, co):
                  name="out-of-range ids are skipped")
 
 
+@pytest.mark.parametrize("n,C,V,hi,dtype,idx_dtype", [
+    (2048, 512, 4095, 3, torch.float32, torch.int32),        # the reference's hot-row case: three ids, 2048 entries
+    (8192, 768, 50257, 50257, torch.bfloat16, torch.int64),   # benchmark shape, ids spread over the table
+    (16384, 1600, 50257, 2000, torch.bfloat16, torch.int64),  # the sort + merge path, segments across windows
+    (5000, 96, 300, 300, torch.float16, torch.int64),
+    (777, 50, 40, 40, torch.float32, torch.int64),            # rows that are not whole vectors: general path
+    (300, 64, 10, 10, torch.float64, torch.int32),
+])
+def test_embedding_backward_scale_grad_by_freq(ops, co, n, C, V, hi, dtype, idx_dtype):
+    """at::embedding_backward(..., scale_grad_by_freq = true) (src/compute/embedding.cpp:147-157): a
+    row's sum divided by the number of entries that name it; segments inside a wave, across the
+    waves of a window and across windows all take their own count."""
+    ids = randint(0, hi, (n,), 700, dtype=idx_dtype)
+    ids[: n // 3] = 1 if hi > 1 else 0  # one id in a third of the entries: a segment over many windows
+    dout = randn((n, C), 701, dtype=dtype)
+    got = ops.embedding_backward(dev(dout), dev(ids), V, scale_grad_by_freq=True)
+    want = co.embedding_backward(dout, ids, V, scale_grad_by_freq=True)
+    tol = {torch.float32: 2e-6, torch.float64: 1e-12}.get(dtype, 1e-6)
+    assert_close(got, want, atol=tol, name="dweight, scaled")
+    assert not torch.equal(got.cpu(), co.embedding_backward(dout, ids, V))  # the option does something
+    # padding row, and += into an existing gradient: only the new part is scaled
+    pad = ops.embedding_backward(dev(dout), dev(ids), V, padding_idx=1, scale_grad_by_freq=True)
+    assert_close(pad, co.embedding_backward(dout, ids, V, padding_idx=1, scale_grad_by_freq=True), atol=tol,
+                 name="dweight, scaled, padding row")
+    base = randn((V, C), 702, dtype=dtype)
+    acc = ops.embedding_backward(dev(dout), dev(ids), V, dweight=dev(base).clone(), scale_grad_by_freq=True)
+    assert_close(acc, co.embedding_backward(dout, ids, V, dweight=base.clone(), scale_grad_by_freq=True),
+                 atol=4 * tol, name="+= of the scaled sums")
+    again = ops.embedding_backward(dev(dout), dev(ids), V, scale_grad_by_freq=True)
+    assert_bit_exact(again, got, "rerun")
+
+
 def test_embedding_backward_random_cases(ops, co):
     """Seeded random shapes around the kernel's internal boundaries (32-entry windows, 4-entry
     waves, 1024-key tiles, the 32/64-bit key switch) with id patterns that stress each level of

@@ -98,6 +98,23 @@ def test_embedding_routine(host, sched, co, dtype):
 
 
 @pytest.mark.gpu
+def test_embedding_scale_grad_by_freq(host, sched, co):
+    # Embedding::Options::scale_grad_by_freq reaches at::embedding_backward in the reference
+    # (src/compute/embedding.cpp:147-157): a row's gradient is the mean over the entries that name it
+    B, T, V, d = 2, 512, 300, 256
+    ids = randint(0, 40, (B, T), 33, dtype=torch.int64)
+    state = host.Embedding.init(sched, V, d, dtype="float32", scale_grad_by_freq=True)
+    host.Embedding.forward(sched, state, up(host, sched, ids))
+    dout = randn((B, T, d), 34)
+    host.Embedding.backward(sched, state, up(host, sched, dout))
+    want = co.embedding_backward(dout, ids, V, scale_grad_by_freq=True)
+    assert_close(down(host, sched, state.grad_weight), want, atol=2e-6, name="scaled grad")
+    host.Embedding.forward(sched, state, up(host, sched, ids))
+    host.Embedding.backward(sched, state, up(host, sched, dout))
+    assert_close(down(host, sched, state.grad_weight), 2 * want, atol=4e-6, name="scaled grad +=")
+
+
+@pytest.mark.gpu
 def test_embedding_inside_autocast_guard(host, sched, co):
     # test/test_autocast.cpp:158-204: fp32 table and fp32 upstream gradient, guard set to bf16;
     # a gather is not an autocast op, so output and gradient stay fp32

@@ -284,6 +284,31 @@ def test_embedding_backward_matches_aten_and_brute_force():
     assert_close(got_pad, ap.embedding_backward(dout, ids, V, 1), atol=2e-5, name="padding_idx")
 
 
+def test_embedding_backward_scaled_by_frequency():
+    """scale_grad_by_freq: against the ATen CPU op the reference calls with that option, and against
+    the closed form (a row's mean over the entries that name it) in float64."""
+    g = torch.Generator().manual_seed(77)
+    V, C = 23, 12
+    ids = torch.randint(0, 6, (5, 40), generator=g)  # few ids, many repeats
+    ids[0, :3] = 20
+    dout = torch.randn((5, 40, C), generator=g)
+    got = co.embedding_backward(dout, ids, V, scale_grad_by_freq=True)
+    assert_close(got, ap.embedding_backward(dout, ids, V, scale_grad_by_freq=True), atol=2e-6, name="ATen, scaled")
+    flat, d = ids.reshape(-1), dout.reshape(-1, C).double()
+    for k in range(V):
+        rows = d[flat == k]
+        want = rows.mean(0) if len(rows) else torch.zeros(C, dtype=torch.float64)
+        assert_close(got[k], want.float(), atol=1e-6, name=f"row {k}: mean of its entries")
+    assert not torch.allclose(got, co.embedding_backward(dout, ids, V))  # the option does something
+    # with a padding row, and added to an existing gradient (only the new part is scaled)
+    pad = co.embedding_backward(dout, ids, V, padding_idx=2, scale_grad_by_freq=True)
+    assert_close(pad, ap.embedding_backward(dout, ids, V, 2, True), atol=2e-6, name="ATen, scaled, padding row")
+    assert pad[2].abs().max() == 0
+    base = torch.randn((V, C), generator=g)
+    assert_close(co.embedding_backward(dout, ids, V, dweight=base.clone(), scale_grad_by_freq=True), base + got, atol=1e-6,
+                 name="+= of the scaled sums")
+
+
 def test_embedding_backward_bf16_uses_fp32_accumulation():
     V, C = 30, 8
     ids = randint(0, 3, (4, 256), 63)

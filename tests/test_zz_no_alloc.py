@@ -94,3 +94,22 @@ def test_static_scratch_rejects_more_rows_than_it_holds():
                                           _capi.F32, _capi.F32, None)
     assert code == _capi.ERR_STATIC_LIMIT
     assert b"scratch" in lib.cs_hip_error_string(code)
+
+
+def test_static_scratch_at_its_row_limit():
+    """The largest call the array takes: its row losses end exactly at the array's last byte."""
+    lib = _capi.load()
+    dev = torch.device("cuda:0")
+    N, V = lib.cs_fused_classifier_static_max_rows(), 8
+    x = randn((N, V), 15, std=2.0, dtype=torch.float32).to(dev)
+    t = randint(0, V, (N,), 16)
+    t[::5] = -100
+    t = t.to(dev)
+    want = _run(lib, False, x, t, V, keep_rows=False, reduction=_capi.REDUCTION_MEAN)
+    got = _run(lib, True, x, t, V, keep_rows=False, reduction=_capi.REDUCTION_MEAN)
+    _same(got, want, "row limit")
+    # and a small call right after it still finds nothing of it
+    x2 = randn((64, 32), 17, dtype=torch.float32).to(dev)
+    t2 = randint(0, 32, (64,), 18).to(dev)
+    _same(_run(lib, True, x2, t2, 32, keep_rows=False, reduction=_capi.REDUCTION_MEAN),
+          _run(lib, False, x2, t2, 32, keep_rows=False, reduction=_capi.REDUCTION_MEAN), "small call after the largest")
