@@ -128,6 +128,10 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 7 + [c_size_t] + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_void_p],
     ),
+    "cs_fused_classifier_weighted": (
+        c_int,
+        [c_void_p] * 8 + [c_size_t] + [c_int64] * 4 + [c_int, c_float, c_int, c_int, c_void_p],
+    ),
     "cs_fused_classifier_static_max_rows": (c_int64, []),
     "cs_fused_classifier_static": (
         c_int,

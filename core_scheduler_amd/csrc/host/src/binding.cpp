@@ -117,7 +117,8 @@ PYBIND11_MODULE(_cs_host, m) {
   {
     using Op = compute::CrossEntropy;
     py::class_<Op::State, std::shared_ptr<Op::State>>(m, "CrossEntropyState")
-        .def("total_weight", [](const Op::State &s) { return as_tensor(s.backward.total_weight); });
+        .def("total_weight", [](const Op::State &s) { return as_tensor(s.backward.total_weight); })
+        .def("set_weight", [](Op::State &s, const Tensor &t) { s.forward.weight = t; });
     auto sub = m.def_submodule("CrossEntropy");
     sub.def("init", [](const Scheduler &s, int reduction, int64_t ignore_index, double label_smoothing,
                        int64_t num_classes) {

@@ -82,7 +82,8 @@ Tensor CrossEntropy::forward(const Scheduler &scheduler, const std::shared_ptr<S
          std::vector<ReadOnlyTensor> in /* weight, input, target */, const State::Args &a)
         : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, args{a} {}
     void operator()() const override {
-      CS_ASSERT_TRUE(!T(input()[0]).defined(), "per-class weights are not supported");
+      // state->forward.weight: nll_loss's per-class weights (src/compute/cross_entropy.cpp:52-55), fp32 for the kernel
+      const at::Tensor cw = T(input()[0]).defined() ? T(input()[0]).to(at::kFloat).contiguous() : at::Tensor{};
       const at::Tensor x = T(input()[1]).contiguous();
       const at::Tensor t = T(input()[2]).contiguous();
       TORCH_CHECK(x.dim() == 2, "CrossEntropy expects [N, C] logits");
@@ -95,11 +96,14 @@ Tensor CrossEntropy::forward(const Scheduler &scheduler, const std::shared_ptr<S
       const auto f32 = x.options().dtype(at::kFloat);
       at::Tensor rows = at::empty({N}, f32), loss = at::empty({}, f32), total = at::empty({}, f32);
       at::Tensor ws = workspace(cs_fused_classifier_workspace_bytes(N), x);
-      check(cs_fused_classifier(x.data_ptr(), grad.data_ptr(), t.data_ptr<int64_t>(), rows.data_ptr<float>(),
-                                loss.data_ptr<float>(), total.data_ptr<float>(), ws.data_ptr(), ws.numel(), N, V,
-                                stride, args.ignore_index, static_cast<int>(args.reduction), 1.f,
-                                dtype_of(x.scalar_type()), dtype_of(g_type), current_stream()),
+      TORCH_CHECK(!cw.defined() || cw.numel() == V, "CrossEntropy: weight must have one entry per class");
+      check(cs_fused_classifier_weighted(x.data_ptr(), grad.data_ptr(), t.data_ptr<int64_t>(),
+                                         cw.defined() ? cw.data_ptr<float>() : nullptr, rows.data_ptr<float>(),
+                                         loss.data_ptr<float>(), total.data_ptr<float>(), ws.data_ptr(), ws.numel(), N,
+                                         V, stride, args.ignore_index, static_cast<int>(args.reduction), 1.f,
+                                         dtype_of(x.scalar_type()), dtype_of(g_type), current_stream()),
             name());
+      if (cw.defined()) intermediate().push_back(cw);
       T(output()[0]) = grad;
       // The reference hands out what nll_loss_forward returns: loss and total weight in the dtype
       // of the log-probabilities (cross_entropy.cpp:57-66), which is 16-bit for 16-bit logits

@@ -51,10 +51,15 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t *__restric
                                                         int64_t N, int64_t V,
                                                         int64_t ignore_index,
                                                         int *__restrict__ ws_count,
-                                                        float *__restrict__ ws_weight) {
+                                                        float *__restrict__ ws_weight,
+                                                        const float *__restrict__ class_weight) {
   __shared__ int scratch[16];
+  __shared__ float wscratch[16];
   const int tid = threadIdx.x;
   int c = 0;
+  float wsum[kSmallInFlight];  // per-class weights of the rows that count: interleaved sums, fixed order
+#pragma unroll
+  for (int u = 0; u < kSmallInFlight; ++u) wsum[u] = 0.f;
   for (int64_t i0 = tid; i0 < N; i0 += (int64_t)1024 * kSmallInFlight) {
     int64_t t[kSmallInFlight];
 #pragma unroll
@@ -64,11 +69,25 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t *__restric
     }
 #pragma unroll
     for (int u = 0; u < kSmallInFlight; ++u) c += target_counts(t[u], V, ignore_index);
+    if (class_weight != nullptr) {  // block-uniform
+      float w[kSmallInFlight];
+#pragma unroll
+      for (int u = 0; u < kSmallInFlight; ++u) w[u] = class_weight[target_counts(t[u], V, ignore_index) ? t[u] : 0];
+#pragma unroll
+      for (int u = 0; u < kSmallInFlight; ++u) wsum[u] += target_counts(t[u], V, ignore_index) ? w[u] : 0.f;
+    }
   }
   c = block_reduce(c, SumOp{}, 0, scratch);
+  float total = (float)c;  // without class weights every row that counts weighs 1
+  if (class_weight != nullptr) {
+    float ws_ = 0.f;
+#pragma unroll
+    for (int u = 0; u < kSmallInFlight; ++u) ws_ += wsum[u];
+    total = block_reduce(ws_, SumOp{}, 0.f, wscratch);
+  }
   if (tid == 0) {
     *ws_count = c;
-    *ws_weight = (float)c;
+    *ws_weight = total;
   }
 }
 
@@ -99,9 +118,10 @@ __global__ __launch_bounds__(1024) void ce_reduce_kernel(const float *__restrict
   for (int u = 0; u < kSmallInFlight; ++u) s += part[u];
   s = block_reduce(s, SumOp{}, 0.f, scratch);
   if (tid == 0) {
-    const int c = *ws_count;
-    if (loss) *loss = reduction == CS_REDUCTION_MEAN ? s / (float)c : s;
-    if (total_weight) *total_weight = (float)c;
+    // the float next to the count: the number of rows that count, or the sum of their class weights
+    const float total = reinterpret_cast<const float *>(ws_count)[1];
+    if (loss) *loss = reduction == CS_REDUCTION_MEAN ? s / total : s;
+    if (total_weight) *total_weight = total;
   }
 }
 
@@ -466,7 +486,7 @@ template <typename T, typename TD, int BLOCK>
 __global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
     const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
     const int *__restrict__ ws_count, int64_t N, int64_t V, int64_t row_stride,
-    int64_t ignore_index, int reduction, float dloss) {
+    int64_t ignore_index, int reduction, float dloss, const float *__restrict__ class_weight) {
   constexpr int VN = Vec16<T>::n;
   constexpr int kWaves = BLOCK / kWave;
   constexpr int kTailLane = 32;  // lanes [0, VN) own head elements, [32, 32 + VN) tail elements
@@ -477,8 +497,11 @@ __global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
   const int wave = tid >> 6;
   const int stride = (int)row_stride;  // the host checks that it fits
   const int vcols = (int)V;
-  float scale = dloss;
-  if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
+  // per-class weights (at::nll_loss's `weight`): a row's loss and gradient are scaled by the
+  // weight of its target, and the mean is over the sum of those weights
+  float scale0 = dloss;
+  if (reduction == CS_REDUCTION_MEAN)
+    scale0 = class_weight ? dloss / reinterpret_cast<const float *>(ws_count)[1] : dloss / (float)(*ws_count);
 
   for (int64_t row = blockIdx.x; row < N; row += gridDim.x) {
     const int64_t tgt = targets[row];
@@ -568,9 +591,12 @@ __global__ __launch_bounds__(BLOCK, 8) void ce_rows_wide_kernel(
     const float ps = lane < kWaves ? red_s[lane] : 0.f;
     const float M2 = wave_reduce(pm, MaxOp{});
     const float S = wave_reduce(pm == -INFINITY ? 0.f : ps * __builtin_amdgcn_exp2f(pm - M2), SumOp{});
+    const float wt = class_weight ? class_weight[tgt] : 1.0f;
+    const float scale = class_weight ? scale0 * wt : scale0;
     if (tid == 0 && row_loss) {
       const float x_t = to_acc(x[tgt]);
-      row_loss[row] = (__builtin_amdgcn_logf(S) - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+      const float l = (__builtin_amdgcn_logf(S) - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+      row_loss[row] = class_weight ? l * wt : l;
     }
     if (!d) continue;
     // ---- sweep 2: p = 2^(x log2e - M2) / S, gradient (p - onehot) * scale
@@ -619,7 +645,7 @@ template <typename T, typename TD>
 __global__ __launch_bounds__(256) void ce_rows_general_kernel(
     const T *__restrict__ logits, TD *__restrict__ dlogits, const int64_t *__restrict__ targets,
     float *__restrict__ row_loss, const int *__restrict__ ws_count, int64_t V, int64_t row_stride,
-    int64_t ignore_index, int reduction, float dloss) {
+    int64_t ignore_index, int reduction, float dloss, const float *__restrict__ class_weight) {
   using U = typename Acc<T>::type;
   __shared__ U scratch[4];
   const int64_t row = blockIdx.x;
@@ -643,10 +669,13 @@ __global__ __launch_bounds__(256) void ce_rows_general_kernel(
   for (int64_t c = threadIdx.x; c < V; c += 256) s += exp((U)to_acc(x[c]) - m);
   s = block_reduce(s, SumOp{}, (U)0, scratch);
   const U lse = m + log(s);
-  if (threadIdx.x == 0 && row_loss) row_loss[row] = (float)(lse - (U)to_acc(x[target]));
+  const U wt = class_weight ? (U)class_weight[target] : (U)1;
+  if (threadIdx.x == 0 && row_loss) row_loss[row] = (float)((lse - (U)to_acc(x[target])) * wt);
   if (!dlogits) return;
   U scale = (U)dloss;
-  if (reduction == CS_REDUCTION_MEAN) scale = (U)dloss / (U)(*ws_count);
+  if (reduction == CS_REDUCTION_MEAN)
+    scale = class_weight ? (U)dloss / (U) reinterpret_cast<const float *>(ws_count)[1] : (U)dloss / (U)(*ws_count);
+  scale *= wt;
   for (int64_t c = threadIdx.x; c < row_stride; c += 256) {
     U o = 0;
     if (c < V) {
@@ -678,33 +707,35 @@ int64_t compute_units() {
 template <typename T, typename TD>
 void launch_wide(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
                  const int *ws_count, int64_t N, int64_t V, int64_t row_stride, int64_t ignore_index,
-                 int reduction, float dloss, hipStream_t s) {
+                 int reduction, float dloss, const float *class_weight, hipStream_t s) {
   const int64_t cus = compute_units();
   const int64_t nvec = row_stride / Vec16<T>::n;
   if (nvec > 256 * kWideU * 2) {
     const dim3 grid((unsigned)(N < 2 * cus ? N : 2 * cus));
     ce_rows_wide_kernel<T, TD, 1024><<<grid, dim3(1024), 0, s>>>(
         (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
-        reduction, dloss);
+        reduction, dloss, class_weight);
   } else {
     const dim3 grid((unsigned)(N < 8 * cus ? N : 8 * cus));
     ce_rows_wide_kernel<T, TD, 256><<<grid, dim3(256), 0, s>>>(
         (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
-        reduction, dloss);
+        reduction, dloss, class_weight);
   }
 }
 
 template <typename T, typename TD>
 int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float *row_loss,
                 const int *ws_count, int64_t N, int64_t V, int64_t row_stride,
-                int64_t ignore_index, int reduction, float dloss, hipStream_t s) {
+                int64_t ignore_index, int reduction, float dloss, const float *class_weight, hipStream_t s) {
   constexpr int VN = Vec16<T>::n;
   const bool base_ok = !std::is_same_v<T, double> && is_aligned16(logits) &&
                        (!dlogits || is_aligned16(dlogits)) && row_stride <= (int64_t(1) << 30);
   const bool vec_ok = base_ok && row_stride % VN == 0;
   const dim3 grid((unsigned)N);
   if constexpr (!std::is_same_v<T, double>) {
-    if (vec_ok) {
+    // per-class weights: the two-sweep kernel (any aligned row) or the general one take them; no
+    // caller of the reference sets them, so the row-in-registers kernels stay as they are
+    if (vec_ok && class_weight == nullptr) {
       const int64_t nvec = row_stride / VN;
 #define CS_CE(BLOCK, VPT)                                                                   \
   ce_rows_kernel<T, TD, BLOCK, VPT><<<grid, dim3(BLOCK), 0, s>>>(                           \
@@ -739,7 +770,7 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         if constexpr (sizeof(T) == 4) CS_CE(1024, 16);
       } else {
         launch_wide<T, TD>(logits, dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
-                           reduction, dloss, s);
+                           reduction, dloss, class_weight, s);
       }
 #undef CS_CE
       return launch_status();
@@ -747,14 +778,14 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
     if (base_ok && sizeof(TD) >= sizeof(T)) {
       // rows that start off a 16-byte boundary: split per row into head, vectors and tail
       launch_wide<T, TD>(logits, dlogits, targets, row_loss, ws_count, N, V, row_stride, ignore_index,
-                         reduction, dloss, s);
+                         reduction, dloss, class_weight, s);
       return launch_status();
     }
   }
   ce_rows_general_kernel<T, TD><<<grid, dim3(256), 0, s>>>((const T *)logits, (TD *)dlogits,
                                                             targets, row_loss, ws_count, V,
                                                             row_stride, ignore_index, reduction,
-                                                            dloss);
+                                                            dloss, class_weight);
   return launch_status();
 }
 
@@ -783,6 +814,7 @@ struct CeArgs {
   int reduction;
   float dloss;
   int dtype, dlogits_dtype;
+  const float *class_weight = nullptr;  // [V] fp32, or NULL: every class weighs 1
 };
 
 int ce_validate(const CeArgs &a) {
@@ -804,7 +836,8 @@ int ce_validate(const CeArgs &a) {
   if (a.N > 0 && (!a.logits || !a.targets)) return CS_ERR_INVALID_ARGUMENT;
   if ((a.logits && !aligned_to(a.logits, es)) || (a.dlogits && !aligned_to(a.dlogits, ds)) ||
       (a.targets && !aligned_to(a.targets, 8)) || (a.row_loss && !aligned_to(a.row_loss, 4)) ||
-      (a.loss && !aligned_to(a.loss, 4)) || (a.total_weight && !aligned_to(a.total_weight, 4)))
+      (a.loss && !aligned_to(a.loss, 4)) || (a.total_weight && !aligned_to(a.total_weight, 4)) ||
+      (a.class_weight && !aligned_to(a.class_weight, 4)))
     return CS_ERR_MISALIGNED;
   if (a.dlogits == a.logits && a.dlogits_dtype != a.dtype) return CS_ERR_INVALID_ARGUMENT;
   return CS_OK;
@@ -822,14 +855,14 @@ int ce_run(const CeArgs &a, int phases, void *stream) {
   float *rows = a.row_loss ? a.row_loss : reinterpret_cast<float *>(ws + kWsHeader);
   if (phases & 1) {
     ce_count_kernel<<<dim3(1), dim3(1024), 0, s>>>(a.targets, a.N, a.V, a.ignore_index, ws_count,
-                                                   ws_weight);
+                                                   ws_weight, a.class_weight);
     st = launch_status();
     if (st != CS_OK) return st;
   }
   if ((phases & 2) && a.N > 0) {
 #define CS_CALL(T, TD)                                                                      \
   st = launch_rows<T, TD>(a.logits, a.dlogits, a.targets, rows, ws_count, a.N, a.V,         \
-                          a.row_stride, a.ignore_index, a.reduction, a.dloss, s)
+                          a.row_stride, a.ignore_index, a.reduction, a.dloss, a.class_weight, s)
     const bool wide = a.dlogits_dtype != a.dtype;
     switch (a.dtype) {
       case CS_F32: CS_CALL(float, float); break;
@@ -871,6 +904,19 @@ extern "C" int cs_fused_classifier(const void *logits, void *dlogits, const int6
   const CeArgs a{logits, dlogits, targets,      row_loss,  loss,  total_weight, workspace,
                  workspace_bytes, N, V, row_stride, ignore_index, reduction, dloss, dtype,
                  dlogits_dtype};
+  return ce_run(a, 1 | 2 | 4, stream);
+}
+
+extern "C" int cs_fused_classifier_weighted(const void *logits, void *dlogits, const int64_t *targets,
+                                            const float *class_weight, float *row_loss, float *loss,
+                                            float *total_weight, void *workspace, size_t workspace_bytes,
+                                            int64_t N, int64_t V, int64_t row_stride, int64_t ignore_index,
+                                            int reduction, float dloss, int dtype, int dlogits_dtype,
+                                            void *stream) {
+  CeArgs a{logits, dlogits, targets,      row_loss,  loss,  total_weight, workspace,
+           workspace_bytes, N, V, row_stride, ignore_index, reduction, dloss, dtype,
+           dlogits_dtype};
+  a.class_weight = class_weight;
   return ce_run(a, 1 | 2 | 4, stream);
 }
 

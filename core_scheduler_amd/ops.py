@@ -509,19 +509,22 @@ def embedding_backward_positions(dout, dwpe=None):
 
 # ------------------------------------------------------- fused classifier
 def fused_classifier(logits, targets, num_classes=None, *, ignore_index=-100, reduction="mean", dloss=1.0,
-                     want_dlogits=True, inplace=False, dlogits_dtype=None):
+                     want_dlogits=True, inplace=False, dlogits_dtype=None, class_weight=None):
     """Softmax cross entropy with its gradient in one pass.
 
     logits [N, stride]; classes are columns [0, num_classes).  Returns
     (loss, row_loss, dlogits, total_weight): loss is 0-d for mean/sum and
     row_loss itself for "none"; dlogits is None unless wanted and is `logits`
-    when inplace.
+    when inplace.  `class_weight` ([num_classes] fp32) weighs every row by its
+    target's class, as nll_loss's `weight`.
     """
-    dev = _dev(logits, targets)
+    dev = _dev(logits, targets, class_weight)
     N, stride = logits.shape
     V = stride if num_classes is None else num_classes
     if targets.dtype != torch.int64 or targets.numel() != N:
         raise ValueError("targets must be int64 [N]")
+    if class_weight is not None and (class_weight.dtype != torch.float32 or class_weight.numel() != V):
+        raise ValueError("class_weight must be fp32 [num_classes]")
     row_loss = torch.empty(N, dtype=torch.float32, device=dev)
     loss = torch.empty((), dtype=torch.float32, device=dev)
     total_weight = torch.empty((), dtype=torch.float32, device=dev)
@@ -534,10 +537,14 @@ def fused_classifier(logits, targets, num_classes=None, *, ignore_index=-100, re
     lib = _capi.load()
     ws_bytes = lib.cs_fused_classifier_workspace_bytes(N)
     ws = _workspace(ws_bytes, dev)
+    tail = (_ptr(ws), ws_bytes, N, V, stride, ignore_index, _REDUCTIONS[reduction], dloss, _dt(logits),
+            _dt(dlogits) if dlogits is not None else _dt(logits), _stream(dev))
     with torch.cuda.device(dev):
-        code = lib.cs_fused_classifier(_ptr(logits), _ptr(dlogits), _ptr(targets), _ptr(row_loss), _ptr(loss),
-                                       _ptr(total_weight), _ptr(ws), ws_bytes, N, V, stride, ignore_index,
-                                       _REDUCTIONS[reduction], dloss, _dt(logits),
-                                       _dt(dlogits) if dlogits is not None else _dt(logits), _stream(dev))
+        if class_weight is None:
+            code = lib.cs_fused_classifier(_ptr(logits), _ptr(dlogits), _ptr(targets), _ptr(row_loss), _ptr(loss),
+                                           _ptr(total_weight), *tail)
+        else:
+            code = lib.cs_fused_classifier_weighted(_ptr(logits), _ptr(dlogits), _ptr(targets), _ptr(class_weight),
+                                                    _ptr(row_loss), _ptr(loss), _ptr(total_weight), *tail)
     _capi.check("cs_fused_classifier", code)
     return (row_loss if reduction == "none" else loss), row_loss, dlogits, total_weight

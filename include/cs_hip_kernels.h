@@ -395,6 +395,23 @@ int cs_fused_classifier(const void *logits, void *dlogits,
                         int reduction, float dloss, int dtype,
                         int dlogits_dtype, void *stream);
 
+/* cs_fused_classifier with at::nll_loss's per-class `weight`
+ * (state->forward.weight, src/compute/cross_entropy.cpp:52-63 and :97-105):
+ * class_weight is [V] fp32; a row's loss and gradient are scaled by the weight
+ * of its target, MEAN divides by the sum of those weights over the rows that
+ * are not ignored, and total_weight returns that sum.  class_weight == NULL is
+ * cs_fused_classifier.  No caller in the reference sets a weight, so this
+ * form takes the two-sweep row kernel for every shape. */
+int cs_fused_classifier_weighted(const void *logits, void *dlogits,
+                                 const int64_t *targets,
+                                 const float *class_weight, float *row_loss,
+                                 float *loss, float *total_weight,
+                                 void *workspace, size_t workspace_bytes,
+                                 int64_t N, int64_t V, int64_t row_stride,
+                                 int64_t ignore_index, int reduction,
+                                 float dloss, int dtype, int dlogits_dtype,
+                                 void *stream);
+
 /* The same call split into its three launches, for callers that want to
  * time or capture them apart, or that already know the row count:
  * phases is a bit set of CS_CE_PHASE_COUNT (write the number of rows that are

@@ -16,24 +16,24 @@ import torch
 aten = torch.ops.aten
 
 
-def cross_entropy_forward(x, target, ignore_index=-100, reduction=1):
-    """src/compute/cross_entropy.cpp:57-63 -> (log_probs, loss, total_weight)"""
+def cross_entropy_forward(x, target, ignore_index=-100, reduction=1, weight=None):
+    """src/compute/cross_entropy.cpp:57-63 -> (log_probs, loss, total_weight); `weight` as :52-55"""
     log_probs = aten.log_softmax(x, 1)
-    loss, total_weight = aten.nll_loss_forward(log_probs, target, None, reduction, ignore_index)
+    loss, total_weight = aten.nll_loss_forward(log_probs, target, weight, reduction, ignore_index)
     return log_probs, loss, total_weight
 
 
-def cross_entropy_backward(log_probs, loss, target, total_weight, ignore_index=-100, reduction=1):
-    """src/compute/cross_entropy.cpp:103-109 -> grad_input"""
-    dnll = aten.nll_loss_backward(torch.ones_like(loss), log_probs, target, None, reduction, ignore_index,
+def cross_entropy_backward(log_probs, loss, target, total_weight, ignore_index=-100, reduction=1, weight=None):
+    """src/compute/cross_entropy.cpp:97-109 -> grad_input"""
+    dnll = aten.nll_loss_backward(torch.ones_like(loss), log_probs, target, weight, reduction, ignore_index,
                                   total_weight)
     return aten._log_softmax_backward_data(dnll, log_probs, 1, log_probs.dtype)
 
 
-def cross_entropy(x, target, ignore_index=-100, reduction=1):
+def cross_entropy(x, target, ignore_index=-100, reduction=1, weight=None):
     """forward then backward, as example/gpt2/gpt2_single_device.cpp:674,693-694"""
-    lp, loss, tw = cross_entropy_forward(x, target, ignore_index, reduction)
-    return loss, cross_entropy_backward(lp, loss, target, tw, ignore_index, reduction), tw
+    lp, loss, tw = cross_entropy_forward(x, target, ignore_index, reduction, weight)
+    return loss, cross_entropy_backward(lp, loss, target, tw, ignore_index, reduction, weight), tw
 
 
 def embedding_forward(weight, indices, padding_idx=-1):

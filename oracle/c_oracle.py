@@ -170,7 +170,7 @@ def embedding_backward_positions(dout, dwpe=None):
 
 
 def cross_entropy(logits, targets, num_classes=None, *, ignore_index=-100, reduction="mean", dloss=1.0,
-                  dlogits_dtype=None):
+                  dlogits_dtype=None, class_weight=None):
     """(loss, row_loss, dlogits, total_weight); loss/row_loss stay wide, dlogits is rounded once."""
     xw, sfx = _wide(logits)
     N, stride = logits.shape
@@ -181,6 +181,7 @@ def cross_entropy(logits, targets, num_classes=None, *, ignore_index=-100, reduc
     tw = torch.zeros((), dtype=xw.dtype)
     d = torch.empty_like(xw)
     red = {"none": 0, "mean": 1, "sum": 2}[reduction]
+    cw = None if class_weight is None else class_weight.to(xw.dtype).contiguous()
     _call("oracle_cross_entropy", sfx, _p(xw), _p(t), _p(row), _p(loss), _p(tw), _p(d), I64(N), I64(V),
-          I64(stride), I64(ignore_index), INT(red), DBL(dloss))
+          I64(stride), I64(ignore_index), INT(red), DBL(dloss), _p(cw) if cw is not None else None)
     return (row if reduction == "none" else loss), row, d.to(dlogits_dtype or logits.dtype), tw

@@ -241,13 +241,17 @@ void FN(oracle_embedding_backward_positions)(const REAL *dout, REAL *dwpe, int64
  * (the GPU library's documented choice; ATen raises instead). */
 void FN(oracle_cross_entropy)(const REAL *logits, const int64_t *targets, REAL *row_loss,
                               REAL *loss, REAL *total_weight, REAL *dlogits, int64_t N, int64_t V,
-                              int64_t stride, int64_t ignore_index, int reduction, double dloss) {
-  int64_t count = 0;
+                              int64_t stride, int64_t ignore_index, int reduction, double dloss,
+                              const REAL *class_weight) {
+  /* class_weight (at::nll_loss's `weight`, src/compute/cross_entropy.cpp:52-63; NULL: all 1):
+   * a row's loss and gradient carry the weight of its target, the mean is over the sum of
+   * those weights, which is also what total_weight returns */
+  double count = 0;
   for (int64_t i = 0; i < N; ++i) {
     const int64_t t = targets[i];
-    if (t != ignore_index && t >= 0 && t < V) ++count;
+    if (t != ignore_index && t >= 0 && t < V) count += class_weight ? (double)class_weight[t] : 1.0;
   }
-  const double scale = reduction == 1 ? dloss / (double)count : dloss;
+  const double scale = reduction == 1 ? dloss / count : dloss;
   double total = 0;
   for (int64_t i = 0; i < N; ++i) {
     const REAL *x = logits + i * stride;
@@ -259,22 +263,23 @@ void FN(oracle_cross_entropy)(const REAL *logits, const int64_t *targets, REAL *
         for (int64_t c = 0; c < stride; ++c) dlogits[i * stride + c] = (REAL)0;
       continue;
     }
+    const double w = class_weight ? (double)class_weight[t] : 1.0;
     double mx = x[0];
     for (int64_t c = 1; c < V; ++c) mx = x[c] > mx ? x[c] : mx;
     double s = 0;
     for (int64_t c = 0; c < V; ++c) s += exp((double)x[c] - mx);
     const double lse = mx + log(s);
-    const double li = lse - (double)x[t];
+    const double li = (lse - (double)x[t]) * w;
     if (row_loss) row_loss[i] = (REAL)li;
     total += li;
     if (dlogits) {
       for (int64_t c = 0; c < stride; ++c) {
         double o = 0;
-        if (c < V) o = (exp((double)x[c] - lse) - (c == t ? 1.0 : 0.0)) * scale;
+        if (c < V) o = (exp((double)x[c] - lse) - (c == t ? 1.0 : 0.0)) * scale * w;
         dlogits[i * stride + c] = (REAL)o;
       }
     }
   }
-  if (loss) *loss = (REAL)(reduction == 1 ? total / (double)count : total);
+  if (loss) *loss = (REAL)(reduction == 1 ? total / count : total);
   if (total_weight) *total_weight = (REAL)count;
 }

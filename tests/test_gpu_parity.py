@@ -613,6 +613,42 @@ def test_layernorm_backward_shapes_without_two_call_form(ops):
         ops.layernorm_backward_rows(x, x, dev(randn(64, 86)), dev(randn(64, 87)), dev(randn(50, 88)))
 
 
+@pytest.mark.parametrize("N,V,stride,dtype,grad_dtype", [
+    (512, 50257, 50304, torch.bfloat16, torch.bfloat16),   # the GPT-2 vocabulary, padded stride
+    (300, 50257, 50257, torch.bfloat16, torch.float32),    # unpadded rows, the autocast combination
+    (1024, 384, 384, torch.float32, torch.float32),        # the reference's test width
+    (77, 1000, 1003, torch.float16, torch.float16),
+    (64, 33, 33, torch.float64, torch.float64),
+])
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+def test_cross_entropy_with_class_weights(ops, co, N, V, stride, dtype, grad_dtype, reduction):
+    """at::nll_loss's per-class `weight` (src/compute/cross_entropy.cpp:52-63, 97-105)."""
+    x = randn((N, stride), 800, std=2.0, dtype=dtype)
+    t = randint(0, V, (N,), 801)
+    t[::11] = -100
+    w = (torch.rand(V, generator=torch.Generator().manual_seed(802)) * 2 + 0.05).float()
+    w[3] = 0.0  # a class that carries no weight at all
+    loss, row, d, tw = ops.fused_classifier(dev(x), dev(t), V, reduction=reduction, class_weight=dev(w),
+                                            dlogits_dtype=grad_dtype)
+    want_loss, want_row, want_d, want_tw = co.cross_entropy(x, t, V, reduction=reduction, class_weight=w,
+                                                            dlogits_dtype=grad_dtype)
+    assert_close(tw.cpu().double(), want_tw.double(), atol=1e-3, name="total weight")
+    assert_close(row.cpu().double(), want_row.double(), atol=2e-5, name="row losses")
+    if reduction != "none":
+        assert_close(loss.cpu().double(), want_loss.double(), atol=2e-5 * (N if reduction == "sum" else 1),
+                     name="loss")
+    atol = {torch.float32: 1e-7, torch.float64: 1e-7}.get(grad_dtype, 1e-7)
+    assert_close(d, want_d, atol=atol, name="dlogits")
+    assert (d.cpu()[:, V:] == 0).all()
+    assert (d.cpu()[t == -100] == 0).all()
+    # all weights 1: the bits of the unweighted call's loss
+    ones = ops.fused_classifier(dev(x), dev(t), V, reduction=reduction, class_weight=dev(torch.ones(V)),
+                                dlogits_dtype=grad_dtype)
+    plain = ops.fused_classifier(dev(x), dev(t), V, reduction=reduction, dlogits_dtype=grad_dtype)
+    assert_close(ones[1], plain[1].cpu(), atol=2e-6, name="weights of 1: row losses of the plain call")
+    assert_close(ones[2], plain[2].cpu(), atol=1e-7, name="weights of 1: gradient of the plain call")
+
+
 # -------------------------------------------------------------- Embedding
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("idx_dtype", [torch.int32, torch.int64])

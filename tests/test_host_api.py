@@ -156,6 +156,26 @@ def test_embedding_with_positions(host, sched, co):
 
 # ------------------------------------------------------------------- CrossEntropy
 @pytest.mark.gpu
+def test_cross_entropy_with_class_weights(host, sched, co):
+    # state->forward.weight goes to nll_loss_forward / backward in the reference
+    # (src/compute/cross_entropy.cpp:52-63,97-105)
+    N, V = 512, 384
+    x = randn((N, V), 40)
+    t = randint(0, V, (N,), 41)
+    t[::9] = -100
+    w = torch.rand(V, generator=torch.Generator().manual_seed(42)) + 0.25
+    state = host.CrossEntropy.init(sched)
+    state.set_weight(up(host, sched, w))
+    loss = host.CrossEntropy.forward(sched, state, up(host, sched, x), up(host, sched, t))
+    dx = host.CrossEntropy.backward(sched, state)
+    loss.wait()
+    want_loss, _, want_dx, want_tw = co.cross_entropy(x, t, class_weight=w)
+    assert_close(down(host, sched, loss).double(), want_loss.double(), atol=1e-5, name="weighted loss")
+    assert_close(down(host, sched, dx), want_dx, atol=1e-9, name="weighted dx")
+
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_cross_entropy_routine(host, sched, co, dtype):
     # test/test_cross_entropy.cpp:69-99: x = rand [B*256, 384] (B smaller here), int64 targets

@@ -264,6 +264,42 @@ def test_embedding_forward_is_atens_gather(dtype, idx_dtype):
                      "gather-add")
 
 
+def test_cross_entropy_with_class_weights():
+    """at::nll_loss's `weight` (src/compute/cross_entropy.cpp:52-63, 97-105): the C restatement against
+    the reference's ATen op sequence called with a weight, and against the closed form in float64."""
+    g = torch.Generator().manual_seed(31)
+    N, V = 37, 11
+    x = torch.randn((N, V), generator=g) * 2
+    t = torch.randint(0, V, (N,), generator=g)
+    t[::6] = -100
+    w = torch.rand(V, generator=g) + 0.1
+    for reduction, code in (("mean", 1), ("sum", 2), ("none", 0)):
+        loss, row, d, tw = co.cross_entropy(x, t, reduction=reduction, class_weight=w)
+        a_loss, a_grad, a_tw = ap.cross_entropy(x, t, reduction=code, weight=w)
+        if reduction != "none":
+            assert_close(loss, a_loss, atol=1e-6, name=f"{reduction}: loss vs ATen")
+            assert_close(d, a_grad, atol=1e-8, name=f"{reduction}: gradient vs ATen")
+            assert_close(tw, a_tw, atol=1e-6, name=f"{reduction}: total weight vs ATen")
+        else:
+            assert_close(row, a_loss, atol=1e-6, name="none: row losses vs ATen")
+    live = t != -100
+    lp = torch.log_softmax(x.double(), 1)
+    wt = torch.where(live, w.double()[t.clamp(min=0)], torch.zeros((), dtype=torch.float64))
+    nll = -lp[torch.arange(N), t.clamp(min=0)] * wt
+    loss, row, d, tw = co.cross_entropy(x, t, class_weight=w)
+    assert_close(tw.double(), wt.sum(), atol=1e-6, name="total weight = sum of the targets' weights")
+    assert_close(loss.double(), nll.sum() / wt.sum(), atol=1e-6, name="weighted mean")
+    onehot = torch.zeros((N, V), dtype=torch.float64)
+    onehot[torch.arange(N)[live], t[live]] = 1
+    want = (lp.exp() - onehot) * (wt / wt.sum())[:, None]
+    assert_close(d.double(), want, atol=1e-8, name="(softmax - onehot) w_t / sum w")
+    # all weights 1 is the unweighted call
+    same = co.cross_entropy(x, t, class_weight=torch.ones(V))
+    plain = co.cross_entropy(x, t)
+    for a, b in zip(same, plain):
+        assert torch.equal(a, b)
+
+
 def test_embedding_backward_matches_aten_and_brute_force():
     # the reference's own case: 2048 contributions over 3 rows (test/test_embedding.cpp:70-72), scaled down
     V, C = 40, 16
