@@ -644,6 +644,62 @@ def per_op_table(args, torch, ops):
     return out
 
 
+def fill_sweep(torch):
+    """The write path on its own: cs_stream_fill_shape over launch shapes and sizes, cold buffers,
+    back-to-back launches between one pair of events.  Prints a table (us per launch, TB/s) on
+    stdout; `python bench.py --fill-sweep` is the whole command."""
+    lib = _capi_lib()
+    dev = torch.device("cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    sizes = [int(x) // 65536 * 65536 for x in (25e6, 77.2e6, 100e6, 400e6, 3.5e9)]
+    pool = torch.empty(int(7.2e9), dtype=torch.uint8, device=dev).zero_()
+
+    def timed(shape, nbytes, reps):
+        nsets = max(2, min(64, int(7e9 // nbytes)))
+        if nsets * nbytes < 6e8:
+            nsets = min(64, int(6e8 // nbytes) + 1)
+
+        def call(i):
+            code = lib.cs_stream_fill_shape(ctypes.c_void_p(pool.data_ptr() + (i % nsets) * nbytes), nbytes, 0, *shape, stream)
+            if code != 0:
+                raise RuntimeError(f"cs_stream_fill_shape{shape}: {code}")
+
+        call(0)
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            hold_gpu(torch, 2.0)
+            e0.record()
+            for i in range(reps):
+                call(i)
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / reps * 1e3)
+        return best
+
+    print("write-only kernel, us per launch and TB/s; lanes x vectors per lane, layout (block: lane-strided chunks, "
+          "wave-KB: whole kilobytes per wave), store, grid (chunks: one chunk per workgroup, k/CU: k persistent workgroups per CU)")
+    print(f"{'lanes':>5s} {'vec':>3s} {'layout':>7s} {'store':>5s} {'grid':>6s} | " + " | ".join(f"{b / 1e6:9.0f} MB" for b in sizes))
+    best = {b: (float("inf"), None) for b in sizes}
+    for plain in (0, 1):
+        for wave_kb in (0, 1):
+            for lanes in (256, 1024):
+                for vec in (1, 2, 4, 8):
+                    for per_cu in ((0, 8) if plain == 0 else (0,)):
+                        shape = (lanes, vec, wave_kb, plain, per_cu)
+                        cells = []
+                        for b in sizes:
+                            us = timed(shape, b, 30 if b < 1e9 else 8)
+                            cells.append(f"{us:7.1f} {b / us / 1e6:4.2f}")
+                            if us < best[b][0]:
+                                best[b] = (us, shape)
+                        print(f"{lanes:5d} {vec:3d} {'wave-KB' if wave_kb else 'block':>7s} {'plain' if plain else 'nt':>5s} "
+                              f"{(str(per_cu) + '/CU') if per_cu else 'chunks':>6s} | " + " | ".join(cells), flush=True)
+    for b in sizes:
+        print(f"fastest at {b / 1e6:.0f} MB: {best[b][0]:.1f} us, (lanes, vectors, wave-KB, plain stores, workgroups per CU) = {best[b][1]}")
+
+
 def cpu_baseline(args, torch):
     """The reference's cross-entropy op sequence on the ATen CPU backend, full configuration-2 size."""
     from oracle import aten_port as ap
@@ -735,6 +791,8 @@ def main():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="K",
                     help="also run K plain 1 GiB copies (to scale hardware traffic counters)")
     ap.add_argument("--full-json", default="", metavar="PATH", help="also write the full per-op table to this file")
+    ap.add_argument("--fill-sweep", action="store_true",
+                    help="only sweep the write-only calibration kernel over launch shapes and print the table")
     ap.add_argument("--cpu-rows", type=int, default=CE_N)
     ap.add_argument("--cpu-reps", type=int, default=5)
     args = ap.parse_args()
@@ -752,6 +810,9 @@ def main():
 
     capi.load()  # raises if the kernel library is not built
     log(f"[bench] device: {torch.cuda.get_device_name(0)}; torch {torch.__version__}")
+    if args.fill_sweep:
+        fill_sweep(torch)
+        return
 
     head = run_headline(args, torch, ops, capi)
     achieved = CE_BYTES / (head["rows_kernel_ms_avg"] * 1e-3) / 1e9

@@ -44,6 +44,7 @@ SIGNATURES = {
     "cs_stream_read_out_words": (c_int64, [c_int64]),
     "cs_stream_read": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "cs_stream_fill": (c_int, [c_void_p, c_int64, ctypes.c_uint32, c_void_p]),
+    "cs_stream_fill_shape": (c_int, [c_void_p, c_int64, ctypes.c_uint32] + [c_int] * 5 + [c_void_p]),
     "cs_stream_update4": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "cs_adamw_step": (c_int, [c_void_p] * 5 + [c_int64, c_int] + [c_double] * 5 + [c_int64, c_void_p]),
     "cs_adamw_multi_table_bytes": (c_size_t, [c_int64]),

@@ -73,7 +73,10 @@ constexpr int kAdamThreads = 256;
 // against 612 us in the other at 124M floats per array; the step gains 3% (620 -> 602 us,
 // 7.96 -> 7.74 ms for 1.56G parameters).
 constexpr int kAdamFlatUnroll = 2;
-constexpr int kAdamMultiUnroll = 4;
+#ifndef CS_ADAM_MULTI_UNROLL
+#define CS_ADAM_MULTI_UNROLL 4
+#endif
+constexpr int kAdamMultiUnroll = CS_ADAM_MULTI_UNROLL;
 
 // Vector index inside a chunk for a lane's u-th access.
 template <int U, bool WAVE_CONTIG>

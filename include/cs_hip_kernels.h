@@ -90,6 +90,18 @@ int cs_stream_copy(void *dst, const void *src, int64_t bytes, void *stream);
 int64_t cs_stream_read_out_words(int64_t bytes);
 int cs_stream_read(const void *src, void *out, int64_t bytes, void *stream);
 int cs_stream_fill(void *dst, int64_t bytes, uint32_t value, void *stream);
+/* cs_stream_fill in a chosen launch shape, for sweeping the write path (the
+ * shape cs_stream_fill uses is the best of these): lanes per workgroup (256
+ * or 1024), 16-byte vectors per lane (1, 2, 4, 8), lane-strided chunks or
+ * (wave_kilobytes != 0) whole kilobytes per wave, nontemporal or
+ * (plain_stores != 0) plain stores, one chunk per workgroup
+ * (workgroups_per_cu == 0) or that many persistent workgroups per CU.
+ * CS_ERR_UNSUPPORTED for a shape that is not built.  No counterpart in the
+ * reference: a measurement aid like cs_stream_copy. */
+int cs_stream_fill_shape(void *dst, int64_t bytes, uint32_t value, int lanes,
+                         int vectors_per_lane, int wave_kilobytes,
+                         int plain_stores, int workgroups_per_cu,
+                         void *stream);
 
 /* A fourth calibration with the memory traffic of the AdamW step and none of
  * its arithmetic: a0..a3 (`bytes` each) are read, a1..a3 rewritten in place
