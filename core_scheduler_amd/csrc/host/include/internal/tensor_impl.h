@@ -10,6 +10,7 @@
 // handle was made.  A consumer on another lane makes its stream wait for the event unless the
 // event has completed already; a consumer on the same lane relies on stream order.
 #pragma once
+#include <memory>
 #include <ATen/core/TensorBody.h>
 
 #include "tensor.h"
@@ -28,6 +29,25 @@ struct ReadOnlyTensor::Impl {
   Event event_;
   auto &event() { return event_; }
   auto &event() const { return event_; }
+
+  // Launches that still have to be enqueued before the tensor holds its value: the column sums
+  // of a LayerNorm backward are added up inside the NEXT LayerNorm backward launch, so until
+  // that launch (or a launch of their own) the weight and bias gradients are only partial rows.
+  // Whoever is about to read or write the tensor - the scheduler for a task's inputs and
+  // outputs, wait() for the host - calls settle() first; it enqueues what is missing on the
+  // stream of the producing task and stamps the tensor with a fresh event.
+  struct Deferred {
+    virtual ~Deferred() = default;
+    virtual void settle() = 0;  // also clears deferred_ of every tensor it completes
+  };
+  std::shared_ptr<Deferred> deferred_;
+  auto &deferred() { return deferred_; }
+  void settle() {
+    if (deferred_) {
+      const auto keep = deferred_;
+      keep->settle();
+    }
+  }
 
   struct {
     bool enable = false;

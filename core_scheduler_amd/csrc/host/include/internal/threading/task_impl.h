@@ -15,6 +15,7 @@
 #pragma once
 #include <ATen/core/TensorBody.h>
 
+#include <memory>
 #include <utility>
 #include <vector>
 
@@ -44,6 +45,10 @@ struct Task::Impl {
   // until the main stream has been made to wait for the task, so the caching allocator cannot
   // hand the blocks to main-stream work while the side stream still uses them.
   [[nodiscard]] auto &intermediate() const { return intermediate_; }
+  // Tensors of EARLIER tasks whose contents this body's launches completed (a LayerNorm backward
+  // adds up the column sums the previous one left).  The body pushes them here; the scheduler
+  // stamps them with this task's lane and event, as it stamps the outputs.
+  [[nodiscard]] auto &completed() const { return completed_; }
   [[nodiscard]] auto &type() const { return type_; }
   [[nodiscard]] auto &priority() const { return priority_; }
 
@@ -55,6 +60,7 @@ struct Task::Impl {
   std::vector<Tensor> output_;
   std::vector<ReadOnlyTensor> input_;
   mutable std::vector<at::Tensor> intermediate_;
+  mutable std::vector<std::shared_ptr<ReadOnlyTensor::Impl>> completed_;
   Priority priority_;
   Type type_;
 };

@@ -4,6 +4,7 @@
 // libcs_hip_kernels.so on the stream the scheduler made current.  There is no ATen compute
 // call on these paths; the init tasks (random / ones / zeros fills) use ATen as the reference does.
 #include <ATen/autocast_mode.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <ATen/ops/empty.h>
 #include <ATen/ops/add.h>
@@ -14,8 +15,11 @@
 #include <ATen/ops/zeros_like.h>
 #include <c10/util/Exception.h>
 
+#include <memory>
+#include <mutex>
 #include <optional>
 #include <string>
+#include <vector>
 
 #include "autocast.h"
 #include "compute/cross_entropy.h"
@@ -28,6 +32,7 @@
 #include "memory/to_torch.h"
 #include "optimizer/adamw.h"
 #include "tensor_impl.h"
+#include "threading/event.h"
 #include "threading/scheduler_impl.h"
 #include "threading/task_impl.h"
 
@@ -64,6 +69,65 @@ at::Tensor workspace(const size_t bytes, const at::Tensor &like) {
 }
 bool autocast_on() { return at::autocast::is_autocast_enabled(at::kCUDA); }
 at::Tensor &T(const ReadOnlyTensor &t) { return t.impl()->tensor(); }
+
+// ---- LayerNorm backward: column sums that ride in the next LayerNorm backward launch
+//
+// A LayerNorm backward launch leaves one fp32 partial row of dgamma and dbeta per workgroup.
+// Adding those rows up is 3 us of work that, as a launch of its own, costs the stream more than
+// that; the kernels can instead add them up in the first workgroups of the NEXT LayerNorm
+// backward launch (cs_layernorm_backward_rows_pending).  A training step runs one backward per
+// norm on the main stream, so only the last norm of the step pays for a launch of its own.
+//
+// Between the two launches the weight and bias gradients are marked (ReadOnlyTensor::Impl::
+// deferred): the scheduler settles a marked tensor before any task that lists it as input or
+// output, and wait() before the host reads it, with a launch of cs_layernorm_backward_finalize
+// on the stream of the backward task.  One record per device is outstanding at a time.
+struct LnSums final : ReadOnlyTensor::Impl::Deferred {
+  at::Tensor partials, dgamma, dbeta;              // dbeta undefined for a norm without bias
+  std::weak_ptr<ReadOnlyTensor::Impl> gw, gb;      // the handles to stamp once the sums are in
+  int64_t C = 0;
+  int x_dtype = 0, p_dtype = 0, accumulate = 0;
+  std::optional<c10::hip::HIPStreamMasqueradingAsCUDA> stream;
+
+  static std::recursive_mutex &mutex() {
+    static auto *m = new std::recursive_mutex;
+    return *m;
+  }
+  // the record of the device, if one is outstanding (never destroyed: it holds device memory,
+  // which must not be released during static teardown)
+  static std::shared_ptr<LnSums> &slot(const int device) {
+    static auto *slots = new std::vector<std::shared_ptr<LnSums>>(64);
+    CS_ASSERT_TRUE(device >= 0 && device < 64, "device index out of range");
+    return (*slots)[static_cast<size_t>(device)];
+  }
+  // the gradients are no longer waiting for this record
+  void detach() {
+    for (const auto &w : {gw, gb})
+      if (const auto impl = w.lock(); impl && impl->deferred().get() == this) impl->deferred().reset();
+    auto &s = slot(stream->device_index());
+    if (s.get() == this) s.reset();
+  }
+  void settle() override {
+    std::lock_guard<std::recursive_mutex> lock{mutex()};
+    if (!partials.defined()) return;  // folded into a launch or settled already
+    const auto keep = slot(stream->device_index());  // detach() may drop the last other owner
+    detach();
+    c10::hip::HIPGuardMasqueradingAsCUDA device_guard{stream->device_index()};
+    c10::hip::HIPStreamGuardMasqueradingAsCUDA stream_guard{*stream};
+    check(cs_layernorm_backward_finalize(partials.data_ptr(), partials.size(0), dgamma.data_ptr(),
+                                         dbeta.defined() ? dbeta.data_ptr() : nullptr, C, x_dtype, p_dtype, accumulate,
+                                         stream->stream()),
+          "cs_layernorm_backward_finalize");
+    Event stamp;
+    stamp.record();
+    for (const auto &w : {gw, gb})
+      if (const auto impl = w.lock()) {
+        impl->priority() = kMain;
+        impl->event() = stamp;
+      }
+    partials = at::Tensor{};
+  }
+};
 }  // namespace
 
 // ============================================================ CrossEntropy
@@ -477,7 +541,9 @@ Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<Sta
   // stream, src/compute/layer_norm.cpp:228-233), and the kernels can be called that way
   // (cs_layernorm_backward_rows / _finalize), but the second kernel is 4 us of work, while making
   // the main stream wait for another stream's event costs it 7 us on this part: at [8192, 768]
-  // the main stream is busy 13.9 us per call with one task and 18.8 us with two.
+  // the main stream is busy 13.9 us per call with one task and 18.8 us with two.  Where the shape
+  // allows, the task launches the row pass only and the column sums ride in the next LayerNorm
+  // backward launch of the stream (LnSums above): 11.3 us per call.
   struct Body final : Task::Impl {
     bool has_bias;
     Body(std::vector<Tensor> out /* dx, grad_weight[, grad_bias] */,
@@ -513,6 +579,14 @@ Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<Sta
         if (has_bias) dbk = *gb;
       }
       const bool kernel_accumulates = accumulate && !widen;
+      if (!widen && rows > 0 && chained(dy, x, mean, rstd, gk, dx, dgk, dbk, kernel_accumulates, rows, C)) {
+        if (!accumulate) {
+          gw = dgk;
+          if (has_bias) *gb = dbk;
+        }
+        T(output()[0]) = dx;
+        return;
+      }
       at::Tensor ws = workspace(cs_layernorm_backward_workspace_bytes(rows, C), x);
       check(cs_layernorm_backward(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), gk.data_ptr(),
                                   dx.data_ptr(), dgk.data_ptr(), has_bias ? dbk.data_ptr() : nullptr, ws.data_ptr(),
@@ -528,6 +602,56 @@ Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<Sta
         if (has_bias) *gb = dbk;
       }
       T(output()[0]) = dx;
+    }
+    // The row pass alone, with the column sums of the previous LayerNorm backward of this stream
+    // added up in the same launch; this call's own sums stay partial rows until the next backward
+    // or until somebody needs the gradients.  False when the shape has no such form.
+    bool chained(const at::Tensor &dy, const at::Tensor &x, const at::Tensor &mean, const at::Tensor &rstd,
+                 const at::Tensor &g, const at::Tensor &dx, const at::Tensor &dg, const at::Tensor &db,
+                 const bool kernel_accumulates, const int64_t rows, const int64_t C) const {
+      const int xt = dtype_of(x.scalar_type()), pt = dtype_of(g.scalar_type());
+      const int64_t n = cs_layernorm_backward_partial_rows(rows, C, xt);
+      if (n <= 0) return false;
+      for (const at::Tensor *t : {&dy, &x, &g, &dx})
+        if (reinterpret_cast<uintptr_t>(t->data_ptr()) % 16 != 0) return false;
+      std::lock_guard<std::recursive_mutex> lock{LnSums::mutex()};
+      const auto here = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+      std::shared_ptr<LnSums> prev = LnSums::slot(here.device_index());
+      if (prev && !(*prev->stream == here && prev->C == C && prev->x_dtype == xt && prev->p_dtype == pt)) {
+        prev->settle();  // another stream, width or type: its sums cannot ride in this launch
+        prev.reset();
+      }
+      at::Tensor partials = at::empty({n, 2, C}, x.options().dtype(at::kFloat));
+      check(cs_layernorm_backward_rows_pending(
+                dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), g.data_ptr(), nullptr, dx.data_ptr(),
+                partials.data_ptr(), static_cast<size_t>(partials.numel()) * 4,
+                prev ? prev->partials.data_ptr() : nullptr, prev ? prev->partials.size(0) : 0,
+                prev ? prev->dgamma.data_ptr() : nullptr,
+                prev && prev->dbeta.defined() ? prev->dbeta.data_ptr() : nullptr, prev ? prev->accumulate : 0, rows, C,
+                dtype_of(dy.scalar_type()), xt, dtype_of(dx.scalar_type()), pt, here.stream()),
+            name());
+      if (prev) {
+        // its gradients are complete with this task: the scheduler stamps them with its event
+        for (const auto &w : {prev->gw, prev->gb})
+          if (const auto impl = w.lock()) completed().push_back(impl);
+        prev->detach();
+        prev->partials = at::Tensor{};
+      }
+      auto mine = std::make_shared<LnSums>();
+      mine->partials = partials;
+      mine->dgamma = dg;
+      if (has_bias) mine->dbeta = db;
+      mine->gw = output()[1].impl();
+      if (has_bias) mine->gb = output()[2].impl();
+      mine->C = C;
+      mine->x_dtype = xt;
+      mine->p_dtype = pt;
+      mine->accumulate = kernel_accumulates ? 1 : 0;
+      mine->stream = here;
+      output()[1].impl()->deferred() = mine;
+      if (has_bias) output()[2].impl()->deferred() = mine;
+      LnSums::slot(here.device_index()) = mine;
+      return true;
     }
     [[nodiscard]] const char *name() const override { return "cs::compute::LayerNorm::backward"; }
   };

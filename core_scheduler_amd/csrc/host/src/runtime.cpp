@@ -100,7 +100,10 @@ TensorOptions ReadOnlyTensor::options() const { return impl_->options(); }
 IntArrayRef ReadOnlyTensor::sizes() const { return impl_->sizes(); }
 int64_t ReadOnlyTensor::size(const int64_t dim) const { return impl_->size(dim); }
 int64_t ReadOnlyTensor::numel() const { return impl_->numel(); }
-void ReadOnlyTensor::wait() const { impl_->event().synchronize(); }
+void ReadOnlyTensor::wait() const {
+  impl_->settle();  // enqueue what the tensor's value still lacks, then wait for all of it
+  impl_->event().synchronize();
+}
 const std::shared_ptr<ReadOnlyTensor::Impl> &ReadOnlyTensor::impl() const { return impl_; }
 void ReadOnlyTensor::reset() { impl_ = std::make_shared<Impl>(); }
 void Tensor::wait() const { ReadOnlyTensor::wait(); }
@@ -181,6 +184,9 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
     // of the inputs that another lane produced, the one stamped last per lane is waited for:
     // a stream finishes its events in the order it recorded them, so that wait covers the rest
     // (each wait is a packet that stalls this stream for microseconds even when it is granted)
+    // tensors whose last launches were put off get them now, before the body reads or rewrites them
+    for (const auto &t : task.impl()->input()) t.impl()->settle();
+    for (const auto &t : task.impl()->output()) t.impl()->settle();
     const Event *latest[Priority::kNumPriority] = {};
     for (const auto &t : task.impl()->input()) {
       const Priority from = t.impl()->priority();
@@ -207,6 +213,11 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
       t.impl()->priority() = lane;
       replace(t.impl()->event(), stamp);
     }
+    for (const auto &done : task.impl()->completed()) {
+      done->priority() = lane;
+      replace(done->event(), stamp);
+    }
+    task.impl()->completed().clear();
     return stamp;
   }
   // one more main task has arrived: side-stream work that is old enough is waited for, unless

@@ -290,6 +290,76 @@ def test_layer_norm_autocast_and_no_bias(host, sched, co):
 
 
 @pytest.mark.gpu
+def test_layer_norm_backward_sums_ride_in_the_next_backward(host, sched):
+    # a step's backward pass: one LayerNorm backward per norm, back to back on the main stream, with
+    # other tasks between them.  Each call leaves its column sums to the next call's launch; the
+    # gradients must hold the bits of the one-call kernel path whenever and however they are read.
+    from core_scheduler_amd import ops
+
+    widths = [768, 768, 1600, 768, 768]  # the width change makes one record settle on its own
+    rows = 2048
+    states, xs, dys, dxs = [], [], [], []
+    for i, C in enumerate(widths):
+        st = host.LayerNorm.init(sched, [C], bias=(i != 3), dtype="float32")
+        st.set_weight(up(host, sched, randn(C, 100 + i, std=0.02, mean=1.0)))
+        if i != 3:
+            st.set_bias(up(host, sched, randn(C, 120 + i, std=0.02)))
+        states.append(st)
+        xs.append(randn((rows, C), 140 + i, dtype=torch.bfloat16))
+        dys.append(randn((rows, C), 160 + i, dtype=torch.bfloat16))
+
+    def want(i, times=1):
+        x, dy = xs[i].to(DEV), dys[i].to(DEV)
+        gamma = down(host, sched, states[i].weight).to(DEV)
+        beta = torch.zeros_like(gamma)
+        _, mean, rstd = ops.layernorm_forward(x, gamma, beta)
+        dx, dg, db = ops.layernorm_backward(dy, x, mean, rstd, gamma)
+        for _ in range(times - 1):
+            ops.layernorm_backward(dy, x, mean, rstd, gamma, dgamma=dg, dbeta=db)
+        return dx.cpu(), dg.cpu(), db.cpu()
+
+    def backward_all():
+        out = []
+        for i, st in enumerate(states):
+            host.LayerNorm.forward(sched, st, up(host, sched, xs[i]))
+        gelu = host.GeLU.init(sched)
+        for i, st in enumerate(states):
+            out.append(host.LayerNorm.backward(sched, st, up(host, sched, dys[i])))
+            host.GeLU.forward(sched, gelu, out[-1])  # an unrelated task between two norms
+        return out
+
+    dxs = backward_all()
+    # read in an order that is not the order of the launches; the last norm's sums had no successor
+    for i in (4, 0, 2, 1, 3):
+        dx2, dg2, db2 = want(i)
+        assert_bit_exact(down(host, sched, states[i].grad_weight), dg2, f"dgamma[{i}]")
+        if i != 3:
+            assert_bit_exact(down(host, sched, states[i].grad_bias), db2, f"dbeta[{i}]")
+        assert_bit_exact(down(host, sched, dxs[i]), dx2, f"dx[{i}]")
+    # a second pass adds to the gradients that exist (micro-batches), again through the chain
+    backward_all()
+    for i in (1, 2, 4):
+        _, dg2, db2 = want(i, times=2)
+        assert_bit_exact(down(host, sched, states[i].grad_weight), dg2, f"dgamma[{i}] +=")
+        assert_bit_exact(down(host, sched, states[i].grad_bias), db2, f"dbeta[{i}] +=")
+    # a task that takes the gradient as its input gets the finished sums without any host read
+    for st in states:
+        st.zero_grad()
+    backward_all()
+    w = up(host, sched, torch.zeros(768))
+    opt = host.AdamW.init(sched, w, lr=1.0, beta1=0.0, beta2=0.0, eps=1.0, weight_decay=0.0, t=0)
+    host.AdamW.step(sched, opt, w, states[4].grad_weight)  # m = g with beta1 = 0
+    assert_bit_exact(down(host, sched, opt.m), want(4)[1], "gradient seen by the optimizer task")
+    # gradients nobody reads are dropped with their sums still outstanding
+    for st in states:
+        st.zero_grad()
+    backward_all()
+    for st in states:
+        st.zero_grad()
+    assert_bit_exact(down(host, sched, backward_all()[0]), want(0)[0], "dx after dropped gradients")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 def test_layer_norm_autocast_with_16_bit_parameters(host, sched, co, dtype):
     # a model whose LayerNorm parameters are 16 bit, run inside the autocast guard: fp32 y, fp32 dy and dx,
