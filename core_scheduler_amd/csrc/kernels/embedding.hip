@@ -323,20 +323,32 @@ __device__ __forceinline__ void positions_block(const T *__restrict__ dout, T *_
 
 // Zero fill of the table, spread over the sort and merge launches, whose own work leaves
 // most CUs idle.  Every row is zeroed before the reduce launch writes the indexed ones.
-// One fill workgroup clears kFillVecs 16-byte vectors.
-#ifndef CS_EMB_FILL_VECS
-#define CS_EMB_FILL_VECS 2048
+// One fill workgroup clears a fixed number of 16-byte vectors, chosen per launch.
+#ifndef CS_EMB_FILL_VECS_RANK
+#define CS_EMB_FILL_VECS_RANK 2048
 #endif
-constexpr int kFillVecs = CS_EMB_FILL_VECS;  // 32 KB: 64 -> 61.6 us at 16384 tokens x 1600 against 128 KB pieces
+#ifndef CS_EMB_FILL_VECS_SORT
+#define CS_EMB_FILL_VECS_SORT 1024
+#endif
+#ifndef CS_EMB_FILL_VECS_MERGE
+#define CS_EMB_FILL_VECS_MERGE 256
+#endif
+// Two vectors per lane next to the ranking workgroups (27.9 us per call against 28.6 with one), one
+// per lane next to the sort and merge workgroups (16384 tokens x 1600: 60.7 us per call against 65.5
+// with 2048 vectors per workgroup in both, 62.7 with 2048 / 256, 62.1 with 1024 / 1024).
+constexpr int kFillVecsRank = CS_EMB_FILL_VECS_RANK;
+constexpr int kFillVecsSort = CS_EMB_FILL_VECS_SORT;
+constexpr int kFillVecsMerge = CS_EMB_FILL_VECS_MERGE;
 #ifndef CS_EMB_FILL_SORT_PCT
-#define CS_EMB_FILL_SORT_PCT 40  // share of the table cleared in the sort launch
+#define CS_EMB_FILL_SORT_PCT 50  // share of the table cleared in the sort launch
 #endif
 
-template <int THREADS>
+template <int THREADS, int kFillVecs>
 __device__ __forceinline__ void zero_fill_block(u32x4 *__restrict__ dst, int64_t vecs, int64_t blk,
                                                 int tid) {
   const u32x4 z = {0u, 0u, 0u, 0u};
   const int64_t v0 = blk * kFillVecs;
+  static_assert(kFillVecs % THREADS == 0, "whole vectors per lane");
 #pragma unroll 8
   for (int u = 0; u < kFillVecs / THREADS; ++u) {
     const int64_t i = v0 + (int64_t)u * THREADS + tid;
@@ -362,7 +374,7 @@ __global__ __launch_bounds__(kTile) void emb_bwd_tile_sort_kernel(
   const int tid = threadIdx.x;
   const int64_t blk = blockIdx.x;
   if (blk > n_tiles + pos_blocks) {
-    zero_fill_block<kTile>(fill_dst, fill_vecs, blk - n_tiles - pos_blocks - 1, tid);
+    zero_fill_block<kTile, kFillVecsSort>(fill_dst, fill_vecs, blk - n_tiles - pos_blocks - 1, tid);
     return;
   }
   if (blk > n_tiles) {
@@ -420,7 +432,7 @@ __global__ __launch_bounds__(kThreads) void emb_bwd_merge_kernel(
   __shared__ u32x4 staged_raw[kMergeChunkBytes / 16];
   const int64_t key_blocks = (int64_t)n_tiles * (kTile / kThreads);
   if ((int64_t)blockIdx.x >= key_blocks) {
-    zero_fill_block<kThreads>(fill_dst, fill_vecs, (int64_t)blockIdx.x - key_blocks, threadIdx.x);
+    zero_fill_block<kThreads, kFillVecsMerge>(fill_dst, fill_vecs, (int64_t)blockIdx.x - key_blocks, threadIdx.x);
     return;
   }
   const KeyT *staged = reinterpret_cast<const KeyT *>(staged_raw);
@@ -517,7 +529,7 @@ __global__ __launch_bounds__(kRankThreads) void emb_bwd_rank_kernel(
   const int tid = threadIdx.x;
   const int64_t blk = blockIdx.x;
   if (blk >= rank_blocks + pos_blocks) {
-    zero_fill_block<kRankThreads>(fill_dst, fill_vecs, blk - rank_blocks - pos_blocks, tid);
+    zero_fill_block<kRankThreads, kFillVecsRank>(fill_dst, fill_vecs, blk - rank_blocks - pos_blocks, tid);
     return;
   }
   if (blk >= rank_blocks) {
@@ -1087,12 +1099,12 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
   const int pos_log2_slices = position_slices(B);
   const int64_t pos_blocks =
       fused_positions ? ceil_div(TC / Vec16<T>::n, (int64_t)(kTile >> pos_log2_slices)) : 0;
-  const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecs);
   const int64_t n_quads = ceil_div(n, (int64_t)4);
   if ((size_t)n_quads * 4 * sizeof(KeyT) <= kRankMaxKeyBytes) {
     // a short list: one launch ranks every key against all others
     static_assert(kRankThreads == kTile, "positions_block assumes kTile lanes");
     const int64_t rank_blocks = ceil_div(n_quads * 4, (int64_t)kRankOwn);
+    const int64_t fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecsRank);
     const int64_t blocks = rank_blocks + pos_blocks + fill_blocks;
     if (blocks == 0) return CS_OK;
     size_t lds = (size_t)n_quads * 4 * sizeof(KeyT) + kRankPartBytes;
@@ -1106,10 +1118,10 @@ int sort_launch(const void *ids, char *ws, const BwdLayout &L, int64_t n, int64_
     return launch_status();
   }
   // whole fill workgroups to the sort launch, the remainder to the merge launch
-  const int64_t sort_fill_blocks = fill_blocks * CS_EMB_FILL_SORT_PCT / 100;
+  const int64_t sort_fill_blocks = ceil_div(fill_vecs, (int64_t)kFillVecsSort) * CS_EMB_FILL_SORT_PCT / 100;
   const int64_t sort_fill_vecs =
-      sort_fill_blocks * kFillVecs < fill_vecs ? sort_fill_blocks * kFillVecs : fill_vecs;
-  const int64_t merge_fill_blocks = fill_blocks - sort_fill_blocks;
+      sort_fill_blocks * kFillVecsSort < fill_vecs ? sort_fill_blocks * kFillVecsSort : fill_vecs;
+  const int64_t merge_fill_blocks = ceil_div(fill_vecs - sort_fill_vecs, (int64_t)kFillVecsMerge);
   const int64_t blocks = L.n_tiles + 1 + pos_blocks + sort_fill_blocks;
   const int64_t mblocks = L.n_tiles * kTile / kThreads + merge_fill_blocks;
   if (blocks > 0x7fffffffLL || mblocks > 0x7fffffffLL) return CS_ERR_TOO_LARGE;
