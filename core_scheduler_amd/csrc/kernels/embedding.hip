@@ -611,6 +611,18 @@ constexpr int kRedWaves = kWindow / kOwn;       // 8
 constexpr int kRedThreads = kRedWaves * kWave;  // 512: two workgroups share a CU
 constexpr int kFinThreads = 1024;               // finish kernel
 constexpr int kFinWaves = kFinThreads / kWave;
+#ifndef CS_EMB_FIN_DIRECT_ROWS
+#define CS_EMB_FIN_DIRECT_ROWS 8
+#endif
+#ifndef CS_EMB_FIN_MAX_GROUPS
+#define CS_EMB_FIN_MAX_GROUPS 8
+#endif
+#ifndef CS_EMB_FIN_IN_FLIGHT
+#define CS_EMB_FIN_IN_FLIGHT 8
+#endif
+constexpr int kFinInFlight = CS_EMB_FIN_IN_FLIGHT;      // rows a lane of a group loads before it adds (a multiple of 8)
+constexpr int kFinDirectRows = CS_EMB_FIN_DIRECT_ROWS;  // segments of up to this many partial rows: one column per lane
+constexpr int kFinMaxGroups = CS_EMB_FIN_MAX_GROUPS;    // lane groups that share the rows of a longer segment
 #ifndef CS_EMB_VPL
 #define CS_EMB_VPL 2
 #endif
@@ -835,37 +847,65 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
     const uint32_t *__restrict__ sorted_id, const float *__restrict__ partial,
     T *__restrict__ dweight, int64_t n, int64_t C, int accumulate, int by_freq) {
   __shared__ int first_other[kFinWaves];
+  __shared__ int first_tail[kFinWaves];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int64_t w = blockIdx.x;
   const int64_t last = w * kWindow + kWindow - 1;
   if (last + 1 >= n) return;  // nothing after this window
-  const uint32_t id = sorted_id[last];
-  if (id == kNoId || sorted_id[last + 1] != id) return;  // no run leaves this window
+  // Everything the decisions below read, and the two partial rows of the usual case (a segment
+  // that ends in the next window), is loaded here at once: taken one after another, each behind
+  // the test of the one before, these were five trips to memory behind the kernel boundary.
+  // Lane t probes window w + 1 + t: its last entry (does the segment leave it?) and its first
+  // (does the segment reach it?).
+  const int64_t pw = w + 1 + tid;
+  const int64_t pq = pw * kWindow + kWindow - 1;
+  uint32_t raw_last = sorted_id[last];
+  uint32_t raw_next = sorted_id[last + 1];
+  uint32_t raw_first = sorted_id[w * kWindow];
+  uint32_t raw_before = sorted_id[w > 0 ? w * kWindow - 1 : 0];
+  uint32_t raw_q = sorted_id[pq < n ? pq : n - 1];
+  uint32_t raw_f = sorted_id[pw * kWindow < n ? pw * kWindow : n - 1];
+  const int64_t col0 = tid < C ? tid : 0;
+  float pre_leave = partial[(w * 2 + 1) * C + col0];        // window w, left over its right edge
+  float pre_enter = partial[((w + 1) * 2 + 0) * C + col0];  // window w + 1, entered over its left edge
+  asm volatile("" : "+v"(raw_last), "+v"(raw_next), "+v"(raw_first), "+v"(raw_before), "+v"(raw_q), "+v"(raw_f),
+                    "+v"(pre_leave), "+v"(pre_enter));
+  const uint32_t id = raw_last;
+  if (id == kNoId || raw_next != id) return;  // no run leaves this window
   // its run began in this window unless the whole window (and the entry before it) has this id
-  if (sorted_id[w * kWindow] == id && w > 0 && sorted_id[w * kWindow - 1] == id) return;
-  // windows after w whose last entry still has this id are left by the segment too; lane t
-  // probes window w + 1 + t, 1024 windows per round
-  int64_t w_hi = -1;  // the window the segment ends in
+  if (raw_first == id && w > 0 && raw_before == id) return;
+  // windows after w whose last entry still has this id are left by the segment too; 1024 windows
+  // per round.  w_hi: the first window whose last entry is not this id.  The segment ends inside
+  // it when its first entry still has the id (`tail`), otherwise at the end of the window before.
+  int64_t w_hi = -1;
+  bool tail = false;
   for (int64_t base = w + 1; w_hi < 0; base += kFinThreads) {
     const int64_t ww = base + tid;
     const int64_t q = ww * kWindow + kWindow - 1;
-    const bool other = q >= n || sorted_id[q] != id;
+    if (base != w + 1) {
+      raw_q = sorted_id[q < n ? q : n - 1];
+      raw_f = sorted_id[ww * kWindow < n ? ww * kWindow : n - 1];
+    }
+    const bool other = q >= n || raw_q != id;
     const uint64_t m = __ballot(other);
-    if (lane == 0) first_other[wave] = m ? __ffsll((long long)m) - 1 : -1;
+    const uint64_t reached = __ballot(ww * kWindow < n && raw_f == id);
+    if (lane == 0) {
+      const int at = m ? __ffsll((long long)m) - 1 : -1;
+      first_other[wave] = at;
+      first_tail[wave] = at >= 0 ? (int)((reached >> at) & 1) : 0;
+    }
     __syncthreads();
     for (int k = 0; k < kFinWaves; ++k) {
       if (first_other[k] >= 0) {
         w_hi = base + k * kWave + first_other[k];
+        tail = first_tail[k] != 0;
         break;
       }
     }
     __syncthreads();
   }
-  // w_hi is the first window whose last entry is not this id.  The segment ends inside it when
-  // its first entry still has the id, otherwise exactly at the end of the window before.
-  const bool tail = w_hi * kWindow < n && sorted_id[w_hi * kWindow] == id;
   const int64_t w_end = tail ? w_hi : w_hi - 1;  // the window the segment ends in (> w)
   // scale_grad_by_freq: the segment's length, from where it begins in window w to where it ends
   // in window w_end (it fills every window in between)
@@ -879,7 +919,70 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
     inv = 1.0f / (float)count;
   }
   T *dst = dweight + (int64_t)id * C;
+  const bool usual = w_end == w + 1;
+  // A hot id (many windows): the partial rows are dealt to groups of lanes, one 16-byte piece of a
+  // row per lane, eight rows in flight per lane; the groups' sums meet in LDS and are added in
+  // group order.  Taken one column per lane instead, the hottest row of a Zipf batch was a chain of
+  // 9-18 trips to memory in a single workgroup while all others had finished.
+  const int64_t rows_in = w_end - w + 1;  // partial rows of the segment
+  const int vc = (int)(C >> 2);           // 16-byte pieces per row
+  if (rows_in > kFinDirectRows && (C & 3) == 0 && vc <= kFinThreads) {
+    __shared__ f32x4 group_sum[kFinThreads];
+    int groups = kFinThreads / vc;
+    if (groups > kFinMaxGroups) groups = kFinMaxGroups;
+    const int g = tid / vc, v = tid - g * vc;
+    if (g < groups) {
+      f32x4 acc[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int64_t r0 = g; r0 < rows_in; r0 += kFinInFlight * groups) {
+        f32x4 x[kFinInFlight];
+#pragma unroll
+        for (int u = 0; u < kFinInFlight; ++u) {
+          const int64_t r = r0 + (int64_t)u * groups;
+          const int64_t rr = r < rows_in ? r : rows_in - 1;
+          // rows before the last were left over the right edge (slot 1), the last was entered (slot 0)
+          const int64_t slot = rr < rows_in - 1 ? (w + rr) * 2 + 1 : w_end * 2;
+          x[u] = *reinterpret_cast<const f32x4 *>(partial + slot * C + 4 * v);
+        }
+#pragma unroll
+        for (int u = 0; u < kFinInFlight; ++u) {
+          const float keep = r0 + (int64_t)u * groups < rows_in ? 1.f : 0.f;
+          acc[u & 7].x = fmaf(x[u].x, keep, acc[u & 7].x);
+          acc[u & 7].y = fmaf(x[u].y, keep, acc[u & 7].y);
+          acc[u & 7].z = fmaf(x[u].z, keep, acc[u & 7].z);
+          acc[u & 7].w = fmaf(x[u].w, keep, acc[u & 7].w);
+        }
+      }
+      f32x4 t;
+      t.x = ((acc[0].x + acc[1].x) + (acc[2].x + acc[3].x)) + ((acc[4].x + acc[5].x) + (acc[6].x + acc[7].x));
+      t.y = ((acc[0].y + acc[1].y) + (acc[2].y + acc[3].y)) + ((acc[4].y + acc[5].y) + (acc[6].y + acc[7].y));
+      t.z = ((acc[0].z + acc[1].z) + (acc[2].z + acc[3].z)) + ((acc[4].z + acc[5].z) + (acc[6].z + acc[7].z));
+      t.w = ((acc[0].w + acc[1].w) + (acc[2].w + acc[3].w)) + ((acc[4].w + acc[5].w) + (acc[6].w + acc[7].w));
+      group_sum[tid] = t;
+    }
+    __syncthreads();
+    if (g == 0) {
+      f32x4 t = group_sum[v];
+      for (int k = 1; k < groups; ++k) {
+        const f32x4 o = group_sum[k * vc + v];
+        t.x += o.x;
+        t.y += o.y;
+        t.z += o.z;
+        t.w += o.w;
+      }
+      const float out[4] = {t.x * inv, t.y * inv, t.z * inv, t.w * inv};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float o = out[k];
+        if (accumulate) o += to_acc(dst[4 * v + k]);
+        dst[4 * v + k] = from_acc<T>(o);
+      }
+    }
+    return;
+  }
   for (int64_t col = tid; col < C; col += kFinThreads) {
+    const bool have = col == tid;  // the first column of the lane came in with the loads above
     // eight interleaved sums keep eight loads in flight; the order is fixed all the same
     float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     int64_t ww = w;
@@ -891,14 +994,17 @@ __global__ __launch_bounds__(kFinThreads) void emb_bwd_finish_kernel(
 #pragma unroll
       for (int u = 0; u < 8; ++u) t[u] += v[u];
     }
-    {
+    if (usual && have) {
+      t[0] += pre_leave;
+      t[7] += pre_enter;
+    } else {
       float v[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) v[u] = ww + u < w_end ? partial[((ww + u) * 2 + 1) * C + col] : 0.f;
 #pragma unroll
       for (int u = 0; u < 7; ++u) t[u] += v[u];  // at most seven windows are left
+      t[7] += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
     }
-    t[7] += partial[(w_end * 2 + 0) * C + col];  // the run that ends there came in over the left edge
     float total = (((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]))) * inv;
     if (accumulate) total += to_acc(dst[col]);
     dst[col] = from_acc<T>(total);
