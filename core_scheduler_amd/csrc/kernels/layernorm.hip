@@ -1228,6 +1228,12 @@ int fwd_typed(const void *x, const void *gamma, const void *beta, void *y, void 
 #ifndef CS_LN_PAIRS
 #define CS_LN_PAIRS 1
 #endif
+#ifndef CS_LN_H3_ALONE_PF
+#define CS_LN_H3_ALONE_PF 1
+#endif
+#ifndef CS_LN_H3_WPE
+#define CS_LN_H3_WPE 2
+#endif
 #ifndef CS_LN_PAIR_PF
 #define CS_LN_PAIR_PF false
 #endif
@@ -1414,6 +1420,9 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
   st = launch_bwd_kernel<TDY, TX, TDX, TP, kLnBwdThreads, 32, VPL, WPE, CS_LN_PAIR_PF, CS_LN_PAIR_KEEP, HAS_DX, \
                          HAS_DP, HAS_DRES>(dy, x, mean, rstd, gamma, dx, workspace, rows, C, dres, pend, blocks, \
                                            lds, s)
+#define CS_LN_K32PF(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                                        \
+  st = launch_bwd_kernel<TDY, TX, TDX, TP, kLnBwdThreads, 32, VPL, WPE, true, CS_LN_PAIR_KEEP, HAS_DX, HAS_DP,   \
+                         HAS_DRES>(dy, x, mean, rstd, gamma, dx, workspace, rows, C, dres, pend, blocks, lds, s)
 #define CS_LN_K64(VPL, WPE, HAS_DX, HAS_DP, HAS_DRES)                                                          \
   st = launch_bwd_kernel<TDY, TX, TDX, TP, CS_LN_W4_THREADS, 64, VPL, WPE, CS_LN_W4_PF, CS_LN_W4_KEEP, HAS_DX,  \
                          HAS_DP, HAS_DRES>(dy, x, mean, rstd, gamma, dx, workspace, rows, C, dres, pend, blocks, \
@@ -1433,7 +1442,16 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
       if (plan.kind == kBwdHalf1) {
         CS_LN_BWD_MASK(CS_LN_K32, 1, 4)
       } else if (plan.kind == kBwdHalf3) {
-        CS_LN_BWD_MASK(CS_LN_K32, 3, 2)
+        // On its own a launch is one workgroup per CU, so a wave may take twice the registers and
+        // load its next two rows while it works on the current ones ([8192,768]: 13.7 -> 13.1 us, with
+        // dresidual 16.1 -> 15.7).  With an earlier call's sums in the launch their workgroups must
+        // fit next to a row workgroup on the same CU, which the larger register budget rules out
+        // (11.3 -> 12.1 us), so that form keeps two workgroups per CU and no prefetch.
+        if (pend.blocks == 0 && dx != nullptr && CS_LN_H3_ALONE_PF) {  // sums alone: 10.9 us without, 11.3 with
+          CS_LN_BWD_MASK(CS_LN_K32PF, 3, 1)
+        } else {
+          CS_LN_BWD_MASK(CS_LN_K32, 3, CS_LN_H3_WPE)
+        }
       } else if (plan.kind == kBwdWave4) {
 #if CS_LN_W4_NEW == 2
         CS_LN_BWD_MASK(CS_LN_K64, 4, CS_LN_W4_WPE)
@@ -1463,6 +1481,7 @@ int bwd_typed(const void *dy, const void *x, const void *mean, const void *rstd,
       }
 #undef CS_LN_BWD_MASK
 #undef CS_LN_K32
+#undef CS_LN_K32PF
 #undef CS_LN_K64
 #undef CS_LN_BWD
       if (st == CS_OK) st = launch_status();
