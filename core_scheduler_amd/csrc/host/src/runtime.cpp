@@ -17,6 +17,7 @@
 #include <deque>
 #include <exception>
 #include <mutex>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -31,17 +32,54 @@
 namespace cs {
 // ------------------------------------------------------------------ events
 struct Event::Impl {
-  void block() { event.block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()); }
+  void block() {
+    settle();
+    event.block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+  }
   void record() {
     static std::atomic<uint64_t> counter{0};
     order = ++counter;
+    stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().id();
+    owed = false;
     event.record();
   }
+  // A record that is made only when somebody needs it.  The scheduler stamps the outputs of a
+  // main-lane task with such an event instead of recording one per task: a record is a packet
+  // between two kernels that keeps the second from starting under the tail of the first (90 tasks
+  // of a GPT-2-small step: 2.19 ms with a record each, 1.92 ms without).  Whoever later waits for
+  // the event (another lane, the host) has it recorded on `home` then, at the stream's tail at
+  // that moment, which covers the task it stands for and whatever the stream got afterwards.
+  void defer(const c10::hip::HIPStreamMasqueradingAsCUDA &on) {
+    home = on;
+    stream = on.id();
+    order = 0;
+    owed = true;
+  }
+  void settle() {
+    if (!owed) return;
+    c10::hip::HIPStreamGuardMasqueradingAsCUDA guard{*home};
+    record();
+  }
+  [[nodiscard]] bool is_owed() const { return owed; }
+  // back to the state of a new event (the pool hands impls out again)
+  void clear() {
+    owed = false;
+    order = 0;
+    stream = -1;
+  }
+  // the stream of the last record(), or the one a deferred record will go to
+  c10::StreamId stream = -1;
   // position of the last record() among all records of the process; 0 = never recorded.
   // Two events recorded on one stream complete in this order.
   uint64_t order = 0;
-  [[nodiscard]] bool query() const { return event.query(); }
-  void synchronize() const { event.synchronize(); }
+  [[nodiscard]] bool query() {
+    settle();
+    return event.query();
+  }
+  void synchronize() {
+    settle();
+    event.synchronize();
+  }
 
  private:
   // Events here order streams of one device and tell the host that work has finished; the data
@@ -51,6 +89,8 @@ struct Event::Impl {
   // with the recorded work for every reader on this device, without the write-back to system
   // scope of a default event (which costs the recording stream ~2.7 us here instead of ~0.9 us).
   at::cuda::CUDAEvent event{hipEventDisableTiming | hipEventReleaseToDevice};
+  std::optional<c10::hip::HIPStreamMasqueradingAsCUDA> home;
+  bool owed = false;
 };
 
 namespace {
@@ -72,6 +112,7 @@ struct EventPool {
     return std::make_shared<Event::Impl>();
   }
   void give(std::shared_ptr<Event::Impl> &&e) {
+    e->clear();
     std::lock_guard<std::mutex> lock{mutex};
     free_list.push_back(std::move(e));
   }
@@ -164,7 +205,7 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
       }
       return;
     }
-    main_done_.block();
+    wait_for(lane, main_done_);
     Parked parked{lane == Priority::kAssist ? kAssistGap : kCommGap, run(task, lane), touched(body)};
     (lane == Priority::kAssist ? assist_ : comm_).push_front(std::move(parked));
   }
@@ -180,35 +221,57 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
   // event is recorded per task (the reference records one per output tensor,
   // src/threading/dynamic_scheduler.cpp:150-160): every output, and the caller's own
   // bookkeeping, share it, since each record is a packet the stream has to work through.
-  static Event run(const Task &task, const Priority lane) {
-    // of the inputs that another lane produced, the one stamped last per lane is waited for:
-    // a stream finishes its events in the order it recorded them, so that wait covers the rest
-    // (each wait is a packet that stalls this stream for microseconds even when it is granted)
+  Event run(const Task &task, const Priority lane) {
     // tensors whose last launches were put off get them now, before the body reads or rewrites them
     for (const auto &t : task.impl()->input()) t.impl()->settle();
     for (const auto &t : task.impl()->output()) t.impl()->settle();
-    const Event *latest[Priority::kNumPriority] = {};
+    // of the inputs that other streams produced, the one stamped last per stream is waited for:
+    // a stream finishes its events in the order it recorded them, so that wait covers the rest
+    // (each wait is a packet that stalls this stream for microseconds even when it is granted)
+    const c10::StreamId here = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().id();
+    constexpr int kMostStreams = 8;
+    const Event *latest[kMostStreams] = {};
+    int n_latest = 0;
     for (const auto &t : task.impl()->input()) {
-      const Priority from = t.impl()->priority();
-      if (from == lane) continue;
       const Event &e = t.impl()->event();
-      if (from >= Priority::kNumPriority) {
+      if (e.impl()->order == 0 && !e.impl()->is_owed()) continue;  // never recorded
+      if (t.impl()->priority() >= Priority::kNumPriority) {
         // handed in from outside, stamped on whatever stream the caller was on: its own wait
         if (!e.query()) e.block();
-      } else if (latest[from] == nullptr || e.impl()->order > latest[from]->impl()->order) {
-        latest[from] = &e;
+        continue;
+      }
+      if (e.impl()->stream == here) continue;  // stream order
+      int k = 0;
+      while (k < n_latest && latest[k]->impl()->stream != e.impl()->stream) ++k;
+      if (k == n_latest) {
+        if (n_latest == kMostStreams) {  // more streams than slots (many schedulers): wait at once
+          wait_for(lane, e);
+          continue;
+        }
+        latest[n_latest++] = &e;
+      } else if (!latest[k]->impl()->is_owed() &&
+                 (e.impl()->is_owed() || e.impl()->order > latest[k]->impl()->order)) {
+        latest[k] = &e;  // an event still owed will be recorded at its stream's tail: it covers the others
       }
     }
-    for (const Event *e : latest) {
-      if (e != nullptr && !e->query()) e->block();
-    }
+    for (int k = 0; k < n_latest; ++k) wait_for(lane, *latest[k]);
     {
       // the task's name as a range in marker traces (rocprofv3 --marker-trace)
       const TraceRange range{task.impl()->name()};
       task();
     }
+    // side-lane tasks get an event of their own; main-lane tasks share one that is recorded when
+    // it is first needed (Event::Impl::defer), and the lane starts another after that
     Event stamp;
-    stamp.record();
+    if (lane == Priority::kMain) {
+      if (!open_.impl()->is_owed()) {
+        open_ = Event{};
+        open_.impl()->defer(streams_[lane]);
+      }
+      stamp = open_;
+    } else {
+      stamp.record();
+    }
     for (const auto &t : task.impl()->output()) {
       t.impl()->priority() = lane;
       replace(t.impl()->event(), stamp);
@@ -222,12 +285,30 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
   }
   // one more main task has arrived: side-stream work that is old enough is waited for, unless
   // it has finished already (a wait costs the main stream about 7 us even then)
-  static void age(std::deque<Parked> &queue) {
+  void age(std::deque<Parked> &queue) {
     for (auto &p : queue) --p.countdown;
     while (!queue.empty() && queue.back().countdown <= 0) {
-      if (!queue.back().done.query()) queue.back().done.block();
+      wait_for(Priority::kMain, queue.back().done);
       queue.pop_back();
     }
+  }
+  // The current stream (the one of `lane`) is made to wait for `e` - unless it already waits for
+  // that event or for a later one recorded on the same stream, which covers it: a stream finishes
+  // its events in the order it recorded them.  A training step's 25 LayerNorm forwards each read
+  // parameters that the optimizer task of the assist lane wrote; one wait serves them all, where
+  // each used to put a wait packet into the main stream (7-18 us of host time apiece while the
+  // optimizer kernel was still running).
+  void wait_for(const Priority lane, const Event &e) {
+    e.impl()->settle();  // an owed record is made now; its position in the stream is known after that
+    const uint64_t order = e.impl()->order;
+    if (order == 0) return;  // never recorded
+    auto &seen = waited_[lane];
+    size_t k = 0;
+    while (k < seen.size() && seen[k].stream != e.impl()->stream) ++k;
+    if (k == seen.size()) seen.push_back({e.impl()->stream, 0});
+    if (order <= seen[k].order) return;  // covered by an earlier wait
+    if (!e.query()) e.block();
+    seen[k].order = order;
   }
   static std::vector<at::Tensor> touched(const Task::Impl &body) {
     std::vector<at::Tensor> keep;
@@ -239,7 +320,15 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
   }
 
   std::vector<Stream> streams_;
+  // per waiting lane and recording stream: position (Event::Impl::order) of the latest event that
+  // the waiting lane's stream has been made to wait for, or has seen completed
+  struct Waited {
+    c10::StreamId stream;
+    uint64_t order;
+  };
+  std::vector<Waited> waited_[Priority::kNumPriority];
   Event main_done_;
+  Event open_;  // the event that main-lane tasks share until somebody needs it
   std::deque<Parked> assist_, comm_;
 };
 }  // namespace

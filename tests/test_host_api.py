@@ -223,6 +223,38 @@ def test_cross_entropy_amp(host, sched, co, dtype):
     assert loss16 == want16.to(x.dtype) or abs(float(loss16) - float(want16)) <= 2.0 ** -7 * float(want16)
 
 
+@pytest.mark.gpu
+def test_host_reads_see_finished_main_lane_work(host, sched):
+    # Main-lane tasks share an event that is recorded only when somebody asks for it.  The asking
+    # is what is tested here: the host reads the output of a long task the moment it is submitted,
+    # with more main-lane work queued behind it, then an assist-lane task (the optimizer) consumes a
+    # main-lane result, and a main-lane task consumes what the optimizer wrote.
+    from core_scheduler_amd import ops
+
+    n = 1 << 25  # 32M elements: ~100 us of kernel time, far longer than the submission
+    state = host.GeLU.init(sched, 1)
+    for seed in (1, 2, 3):
+        x = randn((n,), seed, dtype=torch.bfloat16).to(DEV)
+        y = host.GeLU.forward(sched, state, host.from_torch(sched, x))
+        later = [host.GeLU.forward(sched, state, y) for _ in range(3)]  # queued behind it
+        assert_bit_exact(host.to_torch(sched, y).cpu(), ops.gelu_forward(x, approximate="tanh").cpu(), f"y[{seed}]")
+        assert later[2].defined()
+    # main -> assist -> main
+    w0 = torch.zeros(n // 8, device=DEV)
+    g_src = randn((n // 8,), 9).to(DEV)
+    w = host.from_torch(sched, w0.clone())
+    opt = host.AdamW.init(sched, w, lr=1.0, beta1=0.0, beta2=0.0, eps=1.0, weight_decay=0.0, t=0)
+    gel = host.GeLU.init(sched, 1)
+    grad = host.GeLU.forward(sched, gel, host.from_torch(sched, g_src))   # main lane
+    host.AdamW.step(sched, opt, w, grad)                                  # assist lane, reads grad
+    out = host.GeLU.forward(sched, gel, w)                                # main lane, reads the updated w
+    gref = ops.gelu_forward(g_src, approximate="tanh")
+    wref = w0 - gref / (gref.abs() + 1.0)  # beta1 = beta2 = 0, eps = 1, lr = 1: w -= g / (|g| + 1)
+    assert_close(host.to_torch(sched, w).cpu(), wref.cpu(), atol=1e-6, name="w after the step")
+    assert_close(host.to_torch(sched, out).cpu(), ops.gelu_forward(wref, approximate="tanh").cpu(), atol=1e-6,
+                 name="main-lane task after the step")
+
+
 # ---------------------------------------------------------------------- LayerNorm
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "float64"])
