@@ -641,7 +641,120 @@ def per_op_table(args, torch, ops):
             f"{nbytes/med/1e6/HBM_PEAK_GBPS*100:5.1f}% of HBM peak")
         del opt, w, grad, xs, res, dys, hs, dhs, logits, keep
         torch.cuda.empty_cache()
+
+    # ---- the same step submitted as tasks through the C++ host layer (cs::compute:: /
+    #      cs::optimizer:: calls, three-stream scheduler, Python binding): what a program written
+    #      against the reference's API gets.  The plain ops of that API: LayerNorm without the fused
+    #      residual add, the optimizer as two tasks (fp32 parameters, bf16 tables).  Wall clock
+    #      from the first submission to the host's wait for the last parameter.
+    if wanted("gpt2_small_step_host_layer"):
+        try:
+            from core_scheduler_amd import _cs_host as host
+        except ImportError as e:  # the binding is built by __graft_entry__.build()
+            host = None
+            log(f"[per-op] gpt2_small_step_host_layer skipped: {e}")
+        if host is not None:
+            out.append(host_layer_step(torch, host, g))
+            torch.cuda.empty_cache()
     return out
+
+
+def host_layer_step(torch, host, g):
+    import time
+
+    dev = "cuda:0"
+    B, T, C, L, V = 8, 1024, 768, 12, CE_V
+    rows = B * T
+    sched = host.DynamicScheduler(0)
+
+    def rn(shape, dtype=torch.bfloat16, std=1.0):
+        return torch.empty(shape, device=dev, dtype=torch.float32).normal_(0, std, generator=g).to(dtype)
+
+    def up(t):
+        return host.from_torch(sched, t)
+
+    wte = host.Embedding.init(sched, V, C, dtype="bfloat16")
+    wpe = host.Embedding.init(sched, T, C, dtype="bfloat16")
+    n_ln = 2 * L + 1
+    lns = [host.LayerNorm.init(sched, [C], dtype="float32") for _ in range(n_ln)]
+    gelus = [host.GeLU.init(sched, 1) for _ in range(L)]
+    ids = up(torch.randint(0, V, (B, T), device=dev, generator=g))
+    targets = up(torch.randint(0, V, (rows,), device=dev, generator=g))
+    hs = [up(rn((B, T, 4 * C), std=1.5)) for _ in range(L)]
+    dhs = [up(rn((B, T, 4 * C))) for _ in range(L)]
+    dy_last = up(rn((B, T, C)))
+    logits = [up(rn((rows, CE_STRIDE), std=2.0)) for _ in range(2)]
+    shapes = []
+    for _ in range(L):  # attention and MLP parameters: only the optimizer touches them here
+        shapes += [(3 * C, C), (3 * C,), (C, C), (C,), (4 * C, C), (4 * C,), (C, 4 * C), (C,)]
+    other_w = [up(rn(sh, torch.float32, 0.02)) for sh in shapes]
+    other_g = [up(rn(sh, torch.float32, 1e-3)) for sh in shapes]
+    hp = dict(lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    states = []
+
+    def step(k):
+        h = host.Embedding.forward_with_positions(sched, wte, wpe, ids)
+        for j in range(L):
+            h = host.LayerNorm.forward(sched, lns[2 * j], h)
+            h = host.LayerNorm.forward(sched, lns[2 * j + 1], h)
+            host.GeLU.forward(sched, gelus[j], hs[j])
+        h = host.LayerNorm.forward(sched, lns[2 * L], h)
+        ce = host.CrossEntropy.init(sched, num_classes=V)
+        host.CrossEntropy.forward(sched, ce, logits[k % 2], targets)
+        host.CrossEntropy.backward(sched, ce)
+        d = host.LayerNorm.backward(sched, lns[2 * L], dy_last)
+        for j in reversed(range(L)):
+            host.GeLU.backward(sched, gelus[j], dhs[j])
+            d = host.LayerNorm.backward(sched, lns[2 * j + 1], d)
+            d = host.LayerNorm.backward(sched, lns[2 * j], d)
+        host.Embedding.backward_with_positions(sched, wte, wpe, d)
+        ws, grads = [], []
+        for st in lns:
+            ws += [st.weight, st.bias]
+            grads += [st.grad_weight, st.grad_bias]
+        ws += other_w
+        grads += other_g
+        tabs, tgrads = [wte.weight, wpe.weight], [wte.grad_weight, wpe.grad_weight]
+        if not states:
+            states.append([host.AdamW.init(sched, w, **hp) for w in ws])
+            states.append([host.AdamW.init(sched, w, **hp) for w in tabs])
+        host.AdamW.step_all(sched, states[0], ws, grads)
+        host.AdamW.step_all(sched, states[1], tabs, tgrads)
+        for st in lns:
+            st.zero_grad()
+        wte.zero_grad()
+        wpe.zero_grad()
+        return ws[0]
+
+    for k in range(3):
+        step(k).wait()
+    torch.cuda.synchronize()
+    K, times, submits = 10, [], []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for k in range(K):
+            last = step(k)
+        submits.append((time.perf_counter() - t0) / K)
+        last.wait()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) / K)
+    sec, sub = sorted(times)[1], sorted(submits)[1]
+    ln_f = 2 * rows * C * 2 + 2 * C * 4 + 2 * rows * 4
+    ln_b = 3 * rows * C * 2 + 2 * rows * 4 + 3 * C * 4
+    n_fp32 = n_ln * 2 * C + sum(int(torch.tensor(sh).prod()) for sh in shapes)
+    nbytes = ((rows * C * 2 + rows * 8 + T * C * 2 + rows * C * 2) + n_ln * ln_f
+              + L * 2 * rows * 4 * C * 2 + L * 3 * rows * 4 * C * 2 + 2 * rows * CE_V * 2 + rows * 12 + n_ln * ln_b
+              + rows * C * 2 + V * C * 2 + T * C * 2 + 28 * n_fp32 + 14 * (V * C + T * C))
+    tasks = 1 + n_ln + L + 2 + n_ln + L + 1 + 2
+    ms = sec * 1e3
+    log(f"[per-op] gpt2_small_step_host_layer   {tasks} tasks {ms*1e3:9.1f} us  {nbytes/ms/1e6:8.1f} GB/s  "
+        f"{nbytes/ms/1e6/HBM_PEAK_GBPS*100:5.1f}% of HBM peak  (the host submits a step in {sub*1e6:.0f} us)")
+    return {"op": "gpt2_small_step_host_layer",
+            "config": f"B{B} T{T} C{C} {L} blocks V{V}: {tasks} tasks through the C++ host layer, wall clock",
+            "algorithmic_bytes": nbytes, "ms_warm": round(ms, 5), "ms_cold": round(ms, 5),
+            "gbps_warm": round(nbytes / ms / 1e6, 1), "gbps_cold": round(nbytes / ms / 1e6, 1),
+            "frac_cold": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "buffer_sets": 1, "tasks": tasks,
+            "host_submit_ms": round(sub * 1e3, 4)}
 
 
 def fill_sweep(torch):
