@@ -644,9 +644,10 @@ def per_op_table(args, torch, ops):
 
     # ---- the same step submitted as tasks through the C++ host layer (cs::compute:: /
     #      cs::optimizer:: calls, three-stream scheduler, Python binding): what a program written
-    #      against the reference's API gets.  The plain ops of that API: LayerNorm without the fused
-    #      residual add, the optimizer as two tasks (fp32 parameters, bf16 tables).  Wall clock
-    #      from the first submission to the host's wait for the last parameter.
+    #      against the reference's API gets: the same launches as the row above (LayerNorm through
+    #      the host layer's forward_with_residual / backward_with_residual), the optimizer as two
+    #      tasks (fp32 parameters, bf16 tables).  Wall clock from the first submission to the host's
+    #      wait for the last parameter.
     if wanted("gpt2_small_step_host_layer"):
         try:
             from core_scheduler_amd import _cs_host as host
@@ -683,6 +684,8 @@ def host_layer_step(torch, host, g):
     hs = [up(rn((B, T, 4 * C), std=1.5)) for _ in range(L)]
     dhs = [up(rn((B, T, 4 * C))) for _ in range(L)]
     dy_last = up(rn((B, T, C)))
+    res = [up(rn((B, T, C))) for _ in range(n_ln)]   # what is added to the stream before each norm
+    dres = [up(rn((B, T, C))) for _ in range(n_ln)]  # the gradient that flows past each norm
     logits = [up(rn((rows, CE_STRIDE), std=2.0)) for _ in range(2)]
     shapes = []
     for _ in range(L):  # attention and MLP parameters: only the optimizer touches them here
@@ -694,19 +697,20 @@ def host_layer_step(torch, host, g):
 
     def step(k):
         h = host.Embedding.forward_with_positions(sched, wte, wpe, ids)
+        h = host.LayerNorm.forward(sched, lns[0], h)
+        for j in range(1, n_ln):
+            h, _ = host.LayerNorm.forward_with_residual(sched, lns[j], h, res[j])
         for j in range(L):
-            h = host.LayerNorm.forward(sched, lns[2 * j], h)
-            h = host.LayerNorm.forward(sched, lns[2 * j + 1], h)
             host.GeLU.forward(sched, gelus[j], hs[j])
-        h = host.LayerNorm.forward(sched, lns[2 * L], h)
         ce = host.CrossEntropy.init(sched, num_classes=V)
         host.CrossEntropy.forward(sched, ce, logits[k % 2], targets)
         host.CrossEntropy.backward(sched, ce)
-        d = host.LayerNorm.backward(sched, lns[2 * L], dy_last)
         for j in reversed(range(L)):
             host.GeLU.backward(sched, gelus[j], dhs[j])
-            d = host.LayerNorm.backward(sched, lns[2 * j + 1], d)
-            d = host.LayerNorm.backward(sched, lns[2 * j], d)
+        d = dy_last
+        for j in reversed(range(1, n_ln)):
+            d = host.LayerNorm.backward_with_residual(sched, lns[j], d, dres[j])
+        d = host.LayerNorm.backward(sched, lns[0], d)
         host.Embedding.backward_with_positions(sched, wte, wpe, d)
         ws, grads = [], []
         for st in lns:
@@ -742,8 +746,9 @@ def host_layer_step(torch, host, g):
     ln_f = 2 * rows * C * 2 + 2 * C * 4 + 2 * rows * 4
     ln_b = 3 * rows * C * 2 + 2 * rows * 4 + 3 * C * 4
     n_fp32 = n_ln * 2 * C + sum(int(torch.tensor(sh).prod()) for sh in shapes)
-    nbytes = ((rows * C * 2 + rows * 8 + T * C * 2 + rows * C * 2) + n_ln * ln_f
-              + L * 2 * rows * 4 * C * 2 + L * 3 * rows * 4 * C * 2 + 2 * rows * CE_V * 2 + rows * 12 + n_ln * ln_b
+    nbytes = ((rows * C * 2 + rows * 8 + T * C * 2 + rows * C * 2) + ln_f + (n_ln - 1) * (ln_f + 2 * rows * C * 2)
+              + L * 2 * rows * 4 * C * 2 + L * 3 * rows * 4 * C * 2 + 2 * rows * CE_V * 2 + rows * 12
+              + ln_b + (n_ln - 1) * (ln_b + rows * C * 2)
               + rows * C * 2 + V * C * 2 + T * C * 2 + 28 * n_fp32 + 14 * (V * C + T * C))
     tasks = 1 + n_ln + L + 2 + n_ln + L + 1 + 2
     ms = sec * 1e3

@@ -68,5 +68,19 @@ struct CS_API LayerNorm {
   // main stream more in waiting than the 4 us of summing it would take over).
   static Tensor backward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
                          const ReadOnlyTensor &grad_output);
+
+  // Extensions (no counterpart in the reference's header): the residual stream around a norm
+  // as one task each way.  The reference's GPT-2 block adds and then normalises
+  // (example/gpt2/gpt2_single_device.cpp:459-460) and, going back, differentiates and then adds
+  // (:468-469); the sum and the norm here come out of one kernel with the bits of the two.
+  struct WithResidual {
+    Tensor output;    // LayerNorm(input + residual)
+    Tensor residual;  // input + residual, rounded once to the input's type: the new residual stream
+  };
+  static WithResidual forward_with_residual(const Scheduler &scheduler, const std::shared_ptr<State> &state,
+                                            const ReadOnlyTensor &input, const ReadOnlyTensor &residual);
+  // backward(grad_output) + grad_residual; grad_residual has the shape and type of the result
+  static Tensor backward_with_residual(const Scheduler &scheduler, const std::shared_ptr<State> &state,
+                                       const ReadOnlyTensor &grad_output, const ReadOnlyTensor &grad_residual);
 };
 }  // namespace cs::compute

@@ -154,6 +154,12 @@ PYBIND11_MODULE(_cs_host, m) {
             py::arg("elementwise_affine") = true, py::arg("bias") = true, py::arg("dtype") = "float32");
     sub.def("forward", &Op::forward);
     sub.def("backward", &Op::backward);
+    sub.def("forward_with_residual", [](const Scheduler &s, const std::shared_ptr<Op::State> &state,
+                                        const ReadOnlyTensor &x, const ReadOnlyTensor &residual) {
+      const auto r = Op::forward_with_residual(s, state, x, residual);
+      return std::make_pair(r.output, r.residual);
+    });
+    sub.def("backward_with_residual", &Op::backward_with_residual);
   }
   // ---- Embedding
   {

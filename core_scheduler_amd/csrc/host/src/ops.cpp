@@ -492,181 +492,254 @@ std::shared_ptr<LayerNorm::State> LayerNorm::init(const Scheduler &scheduler, co
                                              options.bias()});
 }
 
-Tensor LayerNorm::forward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
-                          const ReadOnlyTensor &input) {
-  struct Body final : Task::Impl {
-    double eps;
-    bool has_bias;
-    Body(std::vector<Tensor> out /* y, mean, rstd */, std::vector<ReadOnlyTensor> in /* x, weight[, bias] */,
-         const double e, const bool b)
-        : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, eps{e}, has_bias{b} {}
-    void operator()() const override {
-      const at::Tensor x = T(input()[0]).contiguous();
-      const at::Tensor g = T(input()[1]).contiguous();
-      const at::Tensor b = has_bias ? T(input()[2]).contiguous() : at::Tensor{};
-      const int64_t C = x.size(-1), rows = x.numel() / C;
-      TORCH_CHECK(g.numel() == C, "weight does not match the normalised dimension");
-      // native_layer_norm is on ATen's fp32 autocast list: y is fp32 under autocast
-      const auto y_type = (autocast_on() && x.scalar_type() != at::kDouble) ? at::kFloat : x.scalar_type();
-      const auto stat_type = x.scalar_type() == at::kDouble ? at::kDouble : at::kFloat;
-      at::Tensor y = at::empty(x.sizes(), x.options().dtype(y_type));
-      auto stat_sizes = x.sizes().vec();
-      stat_sizes.back() = 1;
-      at::Tensor mean = at::empty(stat_sizes, x.options().dtype(stat_type));
-      at::Tensor rstd = at::empty(stat_sizes, x.options().dtype(stat_type));
+namespace {
+// forward and forward_with_residual: the second takes one more input (after the parameters)
+// and fills one more output (the sum)
+struct LnForwardBody final : Task::Impl {
+  double eps;
+  bool has_bias, has_residual;
+  LnForwardBody(std::vector<Tensor> out /* y, mean, rstd[, sum] */,
+                std::vector<ReadOnlyTensor> in /* x, weight[, bias][, residual] */, const double e, const bool b,
+                const bool r)
+      : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, eps{e}, has_bias{b}, has_residual{r} {}
+  void operator()() const override {
+    const at::Tensor x = T(input()[0]).contiguous();
+    const at::Tensor g = T(input()[1]).contiguous();
+    const at::Tensor b = has_bias ? T(input()[2]).contiguous() : at::Tensor{};
+    const int64_t C = x.size(-1), rows = x.numel() / C;
+    TORCH_CHECK(g.numel() == C, "weight does not match the normalised dimension");
+    // native_layer_norm is on ATen's fp32 autocast list: y is fp32 under autocast
+    const auto y_type = (autocast_on() && x.scalar_type() != at::kDouble) ? at::kFloat : x.scalar_type();
+    const auto stat_type = x.scalar_type() == at::kDouble ? at::kDouble : at::kFloat;
+    at::Tensor y = at::empty(x.sizes(), x.options().dtype(y_type));
+    auto stat_sizes = x.sizes().vec();
+    stat_sizes.back() = 1;
+    at::Tensor mean = at::empty(stat_sizes, x.options().dtype(stat_type));
+    at::Tensor rstd = at::empty(stat_sizes, x.options().dtype(stat_type));
+    if (has_residual) {
+      at::Tensor res = T(input().back()).contiguous();
+      TORCH_CHECK(res.sizes() == x.sizes(), "residual must have the input's shape");
+      if (res.scalar_type() != x.scalar_type()) res = res.to(x.scalar_type());
+      at::Tensor sum = at::empty_like(x);
+      check(cs_add_layernorm_forward(x.data_ptr(), res.data_ptr(), sum.data_ptr(), g.data_ptr(),
+                                     has_bias ? b.data_ptr() : nullptr, y.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                     rows, C, eps, dtype_of(x.scalar_type()), dtype_of(y_type),
+                                     dtype_of(g.scalar_type()), current_stream()),
+            name());
+      T(output()[3]) = sum;
+    } else {
       check(cs_layernorm_forward(x.data_ptr(), g.data_ptr(), has_bias ? b.data_ptr() : nullptr, y.data_ptr(),
                                  mean.data_ptr(), rstd.data_ptr(), rows, C, eps, dtype_of(x.scalar_type()),
                                  dtype_of(y_type), dtype_of(g.scalar_type()), current_stream()),
             name());
-      T(output()[0]) = y;
-      T(output()[1]) = mean;
-      T(output()[2]) = rstd;
     }
-    [[nodiscard]] const char *name() const override { return "cs::compute::LayerNorm::forward"; }
-  };
+    T(output()[0]) = y;
+    T(output()[1]) = mean;
+    T(output()[2]) = rstd;
+  }
+  [[nodiscard]] const char *name() const override {
+    return has_residual ? "cs::compute::LayerNorm::forward_with_residual" : "cs::compute::LayerNorm::forward";
+  }
+};
+}  // namespace
+
+Tensor LayerNorm::forward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
+                          const ReadOnlyTensor &input) {
   Tensor output, mean, rstd;
   std::vector<ReadOnlyTensor> ins{input, state->forward.weight};
   if (state->args.bias) ins.push_back(state->forward.bias);
   state->backward.input = input;
   state->backward.mean = mean;
   state->backward.rstd = rstd;
-  scheduler.impl()->submit(Task{std::make_shared<Body>(std::vector<Tensor>{output, mean, rstd}, std::move(ins),
-                                                        state->args.eps, state->args.bias)});
+  scheduler.impl()->submit(Task{std::make_shared<LnForwardBody>(std::vector<Tensor>{output, mean, rstd}, std::move(ins),
+                                                                 state->args.eps, state->args.bias, false)});
   return output;
 }
 
-Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
-                           const ReadOnlyTensor &grad_output) {
-  // One task on the main stream.  The reference submits two (parameter gradients on the assist
-  // stream, src/compute/layer_norm.cpp:228-233), and the kernels can be called that way
-  // (cs_layernorm_backward_rows / _finalize), but the second kernel is 4 us of work, while making
-  // the main stream wait for another stream's event costs it 7 us on this part: at [8192, 768]
-  // the main stream is busy 13.9 us per call with one task and 18.8 us with two.  Where the shape
-  // allows, the task launches the row pass only and the column sums ride in the next LayerNorm
-  // backward launch of the stream (LnSums above): 11.3 us per call.
-  struct Body final : Task::Impl {
-    bool has_bias;
-    Body(std::vector<Tensor> out /* dx, grad_weight[, grad_bias] */,
-         std::vector<ReadOnlyTensor> in /* grad_output, x, mean, rstd, weight */, const bool b)
-        : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, has_bias{b} {}
-    void operator()() const override {
-      const at::Tensor x = T(input()[1]).contiguous();
-      at::Tensor dy = T(input()[0]).contiguous();
-      const at::Tensor mean = T(input()[2]), rstd = T(input()[3]);
-      const at::Tensor g = T(input()[4]).contiguous();
-      // dy is either x's type or fp32 (autocast over 16-bit x); anything else is brought to x's type
-      const bool narrow_x = x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16;
-      if (dy.scalar_type() != x.scalar_type() && !(narrow_x && dy.scalar_type() == at::kFloat))
-        dy = dy.to(x.scalar_type());
-      const int64_t C = x.size(-1), rows = x.numel() / C;
-      at::Tensor dx = at::empty(x.sizes(), x.options().dtype(dy.scalar_type()));
-      at::Tensor &gw = T(output()[1]);
-      at::Tensor *gb = has_bias ? &T(output()[2]) : nullptr;
-      const bool accumulate = gw.defined();  // += into gradients that already exist
-      if (has_bias) CS_ASSERT_TRUE(gb->defined() == accumulate, "weight and bias gradients must exist together");
-      // fp32 dy with 16-bit parameters (autocast over a model whose LayerNorm weights are 16 bit):
-      // the kernels take fp32 parameters with fp32 dy, so gamma is widened and the parameter
-      // gradients come out in fp32 and are narrowed (or added) afterwards, [C] elements each
-      const bool widen = dy.scalar_type() == at::kFloat && g.scalar_type() != at::kFloat && narrow_x;
-      const at::Tensor gk = widen ? g.to(at::kFloat) : g;
-      at::Tensor dgk, dbk;
-      if (widen || !accumulate) {
-        // an empty batch leaves the gradients untouched: they are zero then
-        dgk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
-        if (has_bias) dbk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
-      } else {
-        dgk = gw;
-        if (has_bias) dbk = *gb;
+LayerNorm::WithResidual LayerNorm::forward_with_residual(const Scheduler &scheduler,
+                                                         const std::shared_ptr<State> &state,
+                                                         const ReadOnlyTensor &input,
+                                                         const ReadOnlyTensor &residual) {
+  Tensor output, mean, rstd, sum;
+  std::vector<ReadOnlyTensor> ins{input, state->forward.weight};
+  if (state->args.bias) ins.push_back(state->forward.bias);
+  ins.push_back(residual);
+  state->backward.input = sum;  // the norm's input is the sum
+  state->backward.mean = mean;
+  state->backward.rstd = rstd;
+  scheduler.impl()->submit(Task{std::make_shared<LnForwardBody>(std::vector<Tensor>{output, mean, rstd, sum},
+                                                                 std::move(ins), state->args.eps, state->args.bias,
+                                                                 true)});
+  return {output, sum};
+}
+
+namespace {
+// One task on the main stream.  The reference submits two (parameter gradients on the assist
+// stream, src/compute/layer_norm.cpp:228-233), and the kernels can be called that way
+// (cs_layernorm_backward_rows / _finalize), but the second kernel is 4 us of work, while making
+// the main stream wait for another stream's event costs it 7 us on this part: at [8192, 768]
+// the main stream is busy 13.9 us per call with one task and 18.8 us with two.  Where the shape
+// allows, the task launches the row pass only and the column sums ride in the next LayerNorm
+// backward launch of the stream (LnSums above): 11.3 us per call.
+struct LnBackwardBody final : Task::Impl {
+  bool has_bias, has_residual;
+  LnBackwardBody(std::vector<Tensor> out /* dx, grad_weight[, grad_bias] */,
+                 std::vector<ReadOnlyTensor> in /* grad_output, x, mean, rstd, weight[, grad_residual] */,
+                 const bool b, const bool r)
+      : Task::Impl{std::move(out), std::move(in), kMain, kCompute}, has_bias{b}, has_residual{r} {}
+  void operator()() const override {
+    const at::Tensor x = T(input()[1]).contiguous();
+    at::Tensor dy = T(input()[0]).contiguous();
+    const at::Tensor mean = T(input()[2]), rstd = T(input()[3]);
+    const at::Tensor g = T(input()[4]).contiguous();
+    // dy is either x's type or fp32 (autocast over 16-bit x); anything else is brought to x's type
+    const bool narrow_x = x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16;
+    if (dy.scalar_type() != x.scalar_type() && !(narrow_x && dy.scalar_type() == at::kFloat))
+      dy = dy.to(x.scalar_type());
+    const int64_t C = x.size(-1), rows = x.numel() / C;
+    at::Tensor dx = at::empty(x.sizes(), x.options().dtype(dy.scalar_type()));
+    // backward_with_residual: the gradient that flows past the norm is added to dx in the same pass
+    at::Tensor dres;
+    if (has_residual) {
+      dres = T(input()[5]).contiguous();
+      TORCH_CHECK(dres.sizes() == x.sizes(), "grad_residual must have the input's shape");
+      if (dres.scalar_type() != dx.scalar_type()) dres = dres.to(dx.scalar_type());
+    }
+    at::Tensor &gw = T(output()[1]);
+    at::Tensor *gb = has_bias ? &T(output()[2]) : nullptr;
+    const bool accumulate = gw.defined();  // += into gradients that already exist
+    if (has_bias) CS_ASSERT_TRUE(gb->defined() == accumulate, "weight and bias gradients must exist together");
+    // fp32 dy with 16-bit parameters (autocast over a model whose LayerNorm weights are 16 bit):
+    // the kernels take fp32 parameters with fp32 dy, so gamma is widened and the parameter
+    // gradients come out in fp32 and are narrowed (or added) afterwards, [C] elements each
+    const bool widen = dy.scalar_type() == at::kFloat && g.scalar_type() != at::kFloat && narrow_x;
+    const at::Tensor gk = widen ? g.to(at::kFloat) : g;
+    at::Tensor dgk, dbk;
+    if (widen || !accumulate) {
+      // an empty batch leaves the gradients untouched: they are zero then
+      dgk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
+      if (has_bias) dbk = rows == 0 ? at::zeros({C}, gk.options()) : at::empty({C}, gk.options());
+    } else {
+      dgk = gw;
+      if (has_bias) dbk = *gb;
+    }
+    const bool kernel_accumulates = accumulate && !widen;
+    if (!widen && rows > 0 && chained(dy, x, mean, rstd, gk, dres, dx, dgk, dbk, kernel_accumulates, rows, C)) {
+      if (!accumulate) {
+        gw = dgk;
+        if (has_bias) *gb = dbk;
       }
-      const bool kernel_accumulates = accumulate && !widen;
-      if (!widen && rows > 0 && chained(dy, x, mean, rstd, gk, dx, dgk, dbk, kernel_accumulates, rows, C)) {
-        if (!accumulate) {
-          gw = dgk;
-          if (has_bias) *gb = dbk;
-        }
-        T(output()[0]) = dx;
-        return;
-      }
-      at::Tensor ws = workspace(cs_layernorm_backward_workspace_bytes(rows, C), x);
+      T(output()[0]) = dx;
+      return;
+    }
+    at::Tensor ws = workspace(cs_layernorm_backward_workspace_bytes(rows, C), x);
+    if (has_residual && rows > 0) {
+      check(cs_layernorm_backward_add(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), gk.data_ptr(),
+                                      dres.data_ptr(), dx.data_ptr(), dgk.data_ptr(),
+                                      has_bias ? dbk.data_ptr() : nullptr, ws.data_ptr(), ws.numel(), rows, C,
+                                      dtype_of(dy.scalar_type()), dtype_of(x.scalar_type()),
+                                      dtype_of(dx.scalar_type()), dtype_of(gk.scalar_type()),
+                                      kernel_accumulates ? 1 : 0, current_stream()),
+            name());
+    } else {
       check(cs_layernorm_backward(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), gk.data_ptr(),
                                   dx.data_ptr(), dgk.data_ptr(), has_bias ? dbk.data_ptr() : nullptr, ws.data_ptr(),
                                   ws.numel(), rows, C, dtype_of(dy.scalar_type()), dtype_of(x.scalar_type()),
                                   dtype_of(dx.scalar_type()), dtype_of(gk.scalar_type()), kernel_accumulates ? 1 : 0,
                                   current_stream()),
             name());
-      if (widen) {
-        gw = accumulate ? gw + dgk.to(g.scalar_type()) : dgk.to(g.scalar_type());
-        if (has_bias) *gb = accumulate ? *gb + dbk.to(g.scalar_type()) : dbk.to(g.scalar_type());
-      } else if (!accumulate) {
-        gw = dgk;
-        if (has_bias) *gb = dbk;
-      }
-      T(output()[0]) = dx;
     }
-    // The row pass alone, with the column sums of the previous LayerNorm backward of this stream
-    // added up in the same launch; this call's own sums stay partial rows until the next backward
-    // or until somebody needs the gradients.  False when the shape has no such form.
-    bool chained(const at::Tensor &dy, const at::Tensor &x, const at::Tensor &mean, const at::Tensor &rstd,
-                 const at::Tensor &g, const at::Tensor &dx, const at::Tensor &dg, const at::Tensor &db,
-                 const bool kernel_accumulates, const int64_t rows, const int64_t C) const {
-      const int xt = dtype_of(x.scalar_type()), pt = dtype_of(g.scalar_type());
-      const int64_t n = cs_layernorm_backward_partial_rows(rows, C, xt);
-      if (n <= 0) return false;
-      for (const at::Tensor *t : {&dy, &x, &g, &dx})
-        if (reinterpret_cast<uintptr_t>(t->data_ptr()) % 16 != 0) return false;
-      std::lock_guard<std::recursive_mutex> lock{LnSums::mutex()};
-      const auto here = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
-      std::shared_ptr<LnSums> prev = LnSums::slot(here.device_index());
-      if (prev && !(*prev->stream == here && prev->C == C && prev->x_dtype == xt && prev->p_dtype == pt)) {
-        prev->settle();  // another stream, width or type: its sums cannot ride in this launch
-        prev.reset();
-      }
-      at::Tensor partials = at::empty({n, 2, C}, x.options().dtype(at::kFloat));
-      check(cs_layernorm_backward_rows_pending(
-                dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), g.data_ptr(), nullptr, dx.data_ptr(),
-                partials.data_ptr(), static_cast<size_t>(partials.numel()) * 4,
-                prev ? prev->partials.data_ptr() : nullptr, prev ? prev->partials.size(0) : 0,
-                prev ? prev->dgamma.data_ptr() : nullptr,
-                prev && prev->dbeta.defined() ? prev->dbeta.data_ptr() : nullptr, prev ? prev->accumulate : 0, rows, C,
-                dtype_of(dy.scalar_type()), xt, dtype_of(dx.scalar_type()), pt, here.stream()),
-            name());
-      if (prev) {
-        // its gradients are complete with this task: the scheduler stamps them with its event
-        for (const auto &w : {prev->gw, prev->gb})
-          if (const auto impl = w.lock()) completed().push_back(impl);
-        prev->detach();
-        prev->partials = at::Tensor{};
-      }
-      auto mine = std::make_shared<LnSums>();
-      mine->partials = partials;
-      mine->dgamma = dg;
-      if (has_bias) mine->dbeta = db;
-      mine->gw = output()[1].impl();
-      if (has_bias) mine->gb = output()[2].impl();
-      mine->C = C;
-      mine->x_dtype = xt;
-      mine->p_dtype = pt;
-      mine->accumulate = kernel_accumulates ? 1 : 0;
-      mine->stream = here;
-      output()[1].impl()->deferred() = mine;
-      if (has_bias) output()[2].impl()->deferred() = mine;
-      LnSums::slot(here.device_index()) = mine;
-      return true;
+    if (widen) {
+      gw = accumulate ? gw + dgk.to(g.scalar_type()) : dgk.to(g.scalar_type());
+      if (has_bias) *gb = accumulate ? *gb + dbk.to(g.scalar_type()) : dbk.to(g.scalar_type());
+    } else if (!accumulate) {
+      gw = dgk;
+      if (has_bias) *gb = dbk;
     }
-    [[nodiscard]] const char *name() const override { return "cs::compute::LayerNorm::backward"; }
-  };
+    T(output()[0]) = dx;
+  }
+  // The row pass alone, with the column sums of the previous LayerNorm backward of this stream
+  // added up in the same launch; this call's own sums stay partial rows until the next backward
+  // or until somebody needs the gradients.  False when the shape has no such form.
+  bool chained(const at::Tensor &dy, const at::Tensor &x, const at::Tensor &mean, const at::Tensor &rstd,
+               const at::Tensor &g, const at::Tensor &dres, const at::Tensor &dx, const at::Tensor &dg,
+               const at::Tensor &db, const bool kernel_accumulates, const int64_t rows, const int64_t C) const {
+    const int xt = dtype_of(x.scalar_type()), pt = dtype_of(g.scalar_type());
+    const int64_t n = cs_layernorm_backward_partial_rows(rows, C, xt);
+    if (n <= 0) return false;
+    for (const at::Tensor *t : {&dy, &x, &g, &dx, &dres})
+      if (t->defined() && reinterpret_cast<uintptr_t>(t->data_ptr()) % 16 != 0) return false;
+    std::lock_guard<std::recursive_mutex> lock{LnSums::mutex()};
+    const auto here = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    std::shared_ptr<LnSums> prev = LnSums::slot(here.device_index());
+    if (prev && !(*prev->stream == here && prev->C == C && prev->x_dtype == xt && prev->p_dtype == pt)) {
+      prev->settle();  // another stream, width or type: its sums cannot ride in this launch
+      prev.reset();
+    }
+    at::Tensor partials = at::empty({n, 2, C}, x.options().dtype(at::kFloat));
+    check(cs_layernorm_backward_rows_pending(
+              dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), g.data_ptr(),
+              dres.defined() ? dres.data_ptr() : nullptr, dx.data_ptr(), partials.data_ptr(), static_cast<size_t>(partials.numel()) * 4,
+              prev ? prev->partials.data_ptr() : nullptr, prev ? prev->partials.size(0) : 0,
+              prev ? prev->dgamma.data_ptr() : nullptr,
+              prev && prev->dbeta.defined() ? prev->dbeta.data_ptr() : nullptr, prev ? prev->accumulate : 0, rows, C,
+              dtype_of(dy.scalar_type()), xt, dtype_of(dx.scalar_type()), pt, here.stream()),
+          name());
+    if (prev) {
+      // its gradients are complete with this task: the scheduler stamps them with its event
+      for (const auto &w : {prev->gw, prev->gb})
+        if (const auto impl = w.lock()) completed().push_back(impl);
+      prev->detach();
+      prev->partials = at::Tensor{};
+    }
+    auto mine = std::make_shared<LnSums>();
+    mine->partials = partials;
+    mine->dgamma = dg;
+    if (has_bias) mine->dbeta = db;
+    mine->gw = output()[1].impl();
+    if (has_bias) mine->gb = output()[2].impl();
+    mine->C = C;
+    mine->x_dtype = xt;
+    mine->p_dtype = pt;
+    mine->accumulate = kernel_accumulates ? 1 : 0;
+    mine->stream = here;
+    output()[1].impl()->deferred() = mine;
+    if (has_bias) output()[2].impl()->deferred() = mine;
+    LnSums::slot(here.device_index()) = mine;
+    return true;
+  }
+  [[nodiscard]] const char *name() const override {
+    return has_residual ? "cs::compute::LayerNorm::backward_with_residual" : "cs::compute::LayerNorm::backward";
+  }
+};
+}  // namespace
+
+namespace {
+Tensor ln_backward(const Scheduler &scheduler, const std::shared_ptr<LayerNorm::State> &state,
+                   const ReadOnlyTensor &grad_output, const ReadOnlyTensor *grad_residual) {
   Tensor grad_input;
   std::vector<Tensor> outs{grad_input, state->forward.grad_weight};
   if (state->args.bias) outs.push_back(state->forward.grad_bias);
-  scheduler.impl()->submit(Task{std::make_shared<Body>(
-      std::move(outs),
-      std::vector<ReadOnlyTensor>{grad_output, state->backward.input, state->backward.mean, state->backward.rstd,
-                                  state->forward.weight},
-      state->args.bias)});
+  std::vector<ReadOnlyTensor> ins{grad_output, state->backward.input, state->backward.mean, state->backward.rstd,
+                                  state->forward.weight};
+  if (grad_residual != nullptr) ins.push_back(*grad_residual);
+  scheduler.impl()->submit(Task{
+      std::make_shared<LnBackwardBody>(std::move(outs), std::move(ins), state->args.bias, grad_residual != nullptr)});
   state->backward.input.reset();
   state->backward.mean.reset();
   state->backward.rstd.reset();
   return grad_input;
+}
+}  // namespace
+
+Tensor LayerNorm::backward(const Scheduler &scheduler, const std::shared_ptr<State> &state,
+                           const ReadOnlyTensor &grad_output) {
+  return ln_backward(scheduler, state, grad_output, nullptr);
+}
+
+Tensor LayerNorm::backward_with_residual(const Scheduler &scheduler, const std::shared_ptr<State> &state,
+                                         const ReadOnlyTensor &grad_output, const ReadOnlyTensor &grad_residual) {
+  return ln_backward(scheduler, state, grad_output, &grad_residual);
 }
 }  // namespace compute
 

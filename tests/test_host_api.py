@@ -392,6 +392,44 @@ def test_layer_norm_backward_sums_ride_in_the_next_backward(host, sched):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("C,rows", [(768, 1024), (1600, 512), (250, 33)])
+def test_layer_norm_with_the_residual_stream(host, sched, C, rows):
+    # example/gpt2/gpt2_single_device.cpp:459-460 (res1 = add(x, attn_out); ln2->forward(res1)) and
+    # :468-469 (dx_ln2 = ln2->backward(dx_mlp); dx_res1 = add(dx_ln2, dx)) as one task each way:
+    # the bits of the separate add and norm tasks
+    x = randn((rows, C), 300, dtype=torch.bfloat16)
+    res = randn((rows, C), 301, dtype=torch.bfloat16)
+    dy = randn((rows, C), 302, dtype=torch.bfloat16)
+    dres = randn((rows, C), 303, dtype=torch.bfloat16)
+    gamma, beta = randn(C, 304, std=0.02, mean=1.0), randn(C, 305, std=0.02)
+
+    def state():
+        st = host.LayerNorm.init(sched, [C], dtype="float32")
+        st.set_weight(up(host, sched, gamma))
+        st.set_bias(up(host, sched, beta))
+        return st
+
+    fused, plain = state(), state()
+    y, new_res = host.LayerNorm.forward_with_residual(sched, fused, up(host, sched, x), up(host, sched, res))
+    total = (x.to(DEV) + res.to(DEV))  # one rounding to bf16, as the kernel does
+    y2 = host.LayerNorm.forward(sched, plain, host.from_torch(sched, total))
+    assert_bit_exact(down(host, sched, new_res), total.cpu(), "x + residual")
+    assert_bit_exact(down(host, sched, y), down(host, sched, y2), "y")
+    dx = host.LayerNorm.backward_with_residual(sched, fused, up(host, sched, dy), up(host, sched, dres))
+    dx2 = host.LayerNorm.backward(sched, plain, up(host, sched, dy))
+    # dx + dresidual in fp32, rounded once (the separate tasks round dx first: up to one bf16 ulp apart)
+    from core_scheduler_amd import ops
+
+    _, mean, rstd = ops.layernorm_forward(total, gamma.to(DEV), beta.to(DEV))
+    want, _, _ = ops.layernorm_backward(dy.to(DEV), total, mean, rstd, gamma.to(DEV), dresidual=dres.to(DEV))
+    assert_bit_exact(down(host, sched, dx), want.cpu(), "dx + dresidual")
+    two_tasks = down(host, sched, dx2).float() + dres.float()
+    assert_close(down(host, sched, dx).float(), two_tasks, atol=0.04, name="against the two tasks")  # bf16 ulp at |v| ~ 4
+    assert_bit_exact(down(host, sched, fused.grad_weight), down(host, sched, plain.grad_weight), "dgamma")
+    assert_bit_exact(down(host, sched, fused.grad_bias), down(host, sched, plain.grad_bias), "dbeta")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["bfloat16", "float16"])
 def test_layer_norm_autocast_with_16_bit_parameters(host, sched, co, dtype):
     # a model whose LayerNorm parameters are 16 bit, run inside the autocast guard: fp32 y, fp32 dy and dx,
