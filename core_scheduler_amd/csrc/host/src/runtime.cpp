@@ -262,16 +262,7 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
     }
     // side-lane tasks get an event of their own; main-lane tasks share one that is recorded when
     // it is first needed (Event::Impl::defer), and the lane starts another after that
-    Event stamp;
-    if (lane == Priority::kMain) {
-      if (!open_.impl()->is_owed()) {
-        open_ = Event{};
-        open_.impl()->defer(streams_[lane]);
-      }
-      stamp = open_;
-    } else {
-      stamp.record();
-    }
+    const Event stamp = lane == Priority::kMain ? shared_stamp() : recorded_stamp();
     for (const auto &t : task.impl()->output()) {
       t.impl()->priority() = lane;
       replace(t.impl()->event(), stamp);
@@ -281,6 +272,18 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
       replace(done->event(), stamp);
     }
     task.impl()->completed().clear();
+    return stamp;
+  }
+  Event shared_stamp() {
+    if (!open_.impl()->is_owed()) {
+      replace(open_, Event{});
+      open_.impl()->defer(streams_[Priority::kMain]);
+    }
+    return open_;
+  }
+  static Event recorded_stamp() {
+    Event stamp;
+    stamp.record();
     return stamp;
   }
   // one more main task has arrived: side-stream work that is old enough is waited for, unless
