@@ -309,11 +309,14 @@ __device__ __forceinline__ float widen(const VecE<T, EPV> &v, int k) {
 // e = 2^((x - m_lane) log2e) is kept in registers, one exchange of (max, sum)
 // pairs across the 16 waves gives the row's max and sum, and the output is
 // e * f with one per-lane factor f = 2^(m_lane*log2e - log2(sum) - max*log2e) * scale.
-template <typename T, typename TD, int VPT, int EPV>
+//
+// HAS_W: per-class weights (nll_loss's `weight`): a row's gradient and loss carry w[target], and
+// the mean divides by the sum of those weights, which the count launch left next to the count.
+template <typename T, typename TD, int VPT, int EPV, bool HAS_W>
 __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     const T *logits, TD *dlogits, const int64_t *__restrict__ targets, float *__restrict__ row_loss,
     const int *__restrict__ ws_count, int64_t N, int64_t V, int64_t row_stride,
-    int64_t ignore_index, int reduction, float dloss) {
+    int64_t ignore_index, int reduction, float dloss, const float *__restrict__ class_weight) {
   constexpr int BLOCK = 1024;
   constexpr int VN = EPV;  // elements per lane per access
   constexpr int kWaves = BLOCK / kWave;
@@ -324,20 +327,21 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
   const int nvec = (int)(row_stride / VN);
   const int iV = (int)V;
 
-  float scale = dloss;
-  if (reduction == CS_REDUCTION_MEAN) scale = dloss / (float)(*ws_count);
-  const float log2_scale = __builtin_amdgcn_logf(fabsf(scale));  // -inf for 0: every output 0
-  const bool negate = scale < 0.f;
+  float scale0 = dloss;
+  if (reduction == CS_REDUCTION_MEAN)
+    scale0 = HAS_W ? dloss / reinterpret_cast<const float *>(ws_count)[1] : dloss / (float)(*ws_count);
+  const float log2_scale0 = __builtin_amdgcn_logf(fabsf(scale0));  // -inf for 0: every output 0
 
   int64_t row = blockIdx.x;
   VecE<T, EPV> cur[VPT];
   int64_t tgt = 0;
   bool live = false;
-  float x_t = 0.f;
+  float x_t = 0.f, wt = 1.f;
   if (row < N) {
     tgt = targets[row];
     live = target_counts(tgt, V, ignore_index);
     if (live) {
+      if constexpr (HAS_W) wt = class_weight[tgt];
       const T *x = logits + row * row_stride;
 #pragma unroll
       for (int j = 0; j < VPT; ++j) {
@@ -354,11 +358,12 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     VecE<T, EPV> nxt[VPT];
     int64_t ntgt = 0;
     bool nlive = false;
-    float nx_t = 0.f;
+    float nx_t = 0.f, nwt = 1.f;
     if (nrow < N) {
       ntgt = targets[nrow];
       nlive = target_counts(ntgt, V, ignore_index);
       if (nlive) {
+        if constexpr (HAS_W) nwt = class_weight[ntgt];
         const T *x = logits + nrow * row_stride;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
@@ -430,7 +435,14 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
       const float log2_S = __builtin_amdgcn_logf(S);
       // loss = ln(sum exp(x - max)) - (x_t - max), the difference to the maximum formed with one
       // fused multiply-add against the rounded M2 the sum was taken with
-      if (tid == 0 && row_loss) row_loss[row] = (log2_S - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+      {
+        const float l = (log2_S - __builtin_fmaf(x_t, kLog2e, -M2)) * kLn2;
+        if (tid == 0 && row_loss) row_loss[row] = HAS_W ? l * wt : l;
+      }
+      // the row's scale: the call's, times the weight of the row's class
+      const float scale = HAS_W ? scale0 * wt : scale0;
+      const float log2_scale = HAS_W ? log2_scale0 + __builtin_amdgcn_logf(fabsf(wt)) : log2_scale0;
+      const bool negate = scale < 0.f;
 
       if (dlogits) {
         // a lane that holds no class column has e = 0 everywhere; give it f = 0 so that
@@ -465,6 +477,7 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     live = nlive;
     tgt = ntgt;
     x_t = nx_t;
+    wt = nwt;
     row = nrow;
   }
 }
@@ -733,9 +746,13 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
   const bool vec_ok = base_ok && row_stride % VN == 0;
   const dim3 grid((unsigned)N);
   if constexpr (!std::is_same_v<T, double>) {
-    // per-class weights: the two-sweep kernel (any aligned row) or the general one take them; no
-    // caller of the reference sets them, so the row-in-registers kernels stay as they are
-    if (vec_ok && class_weight == nullptr) {
+    // per-class weights: the streaming kernel, the two-sweep kernel (any aligned row) and the
+    // general one take them; the small row-in-registers kernels do not (no caller of the reference
+    // sets weights), so weighted calls on narrow rows go to the two-sweep kernel
+    const int64_t nvec_all = row_stride / VN;
+    const bool streams = nvec_all > 256 * 8 &&
+                         nvec_all <= (sizeof(T) == 4 ? 1024 * 8 : sizeof(TD) == 4 ? 512 * 13 : 1024 * 7);
+    if (vec_ok && (class_weight == nullptr || streams)) {
       const int64_t nvec = row_stride / VN;
 #define CS_CE(BLOCK, VPT)                                                                   \
   ce_rows_kernel<T, TD, BLOCK, VPT><<<grid, dim3(BLOCK), 0, s>>>(                           \
@@ -751,10 +768,16 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         // two-sweep kernel and are not built.
         const int64_t cus = compute_units();
         const dim3 pgrid((unsigned)(N < cus ? N : cus));
-#define CS_CE_STREAM(VPT, EPV)                                                              \
-  ce_rows_stream_kernel<T, TD, VPT, EPV><<<pgrid, dim3(1024), 0, s>>>(                      \
-      (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,      \
-      ignore_index, reduction, dloss)
+#define CS_CE_STREAM(VPT, EPV)                                                                    \
+  if (class_weight != nullptr) {                                                                  \
+    ce_rows_stream_kernel<T, TD, VPT, EPV, true><<<pgrid, dim3(1024), 0, s>>>(                    \
+        (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,          \
+        ignore_index, reduction, dloss, class_weight);                                            \
+  } else {                                                                                        \
+    ce_rows_stream_kernel<T, TD, VPT, EPV, false><<<pgrid, dim3(1024), 0, s>>>(                   \
+        (const T *)logits, (TD *)dlogits, targets, row_loss, ws_count, N, V, row_stride,          \
+        ignore_index, reduction, dloss, nullptr);                                                 \
+  }
         if constexpr (sizeof(T) == 2 && sizeof(TD) == 4) {
           CS_CE_STREAM(13, 4);  // 16-bit logits, fp32 gradients (autocast): 4 elements per lane per access
         } else if (nvec <= 1024 * 4) {
@@ -762,7 +785,9 @@ int launch_rows(const void *logits, void *dlogits, const int64_t *targets, float
         } else if (nvec <= 1024 * 7) {
           CS_CE_STREAM(7, VN);
         } else {
-          if constexpr (sizeof(T) == 4) CS_CE_STREAM(8, VN);
+          if constexpr (sizeof(T) == 4) {
+            CS_CE_STREAM(8, VN);
+          }
         }
 #undef CS_CE_STREAM
       } else if (sizeof(T) == 4 && nvec <= 1024 * 16) {

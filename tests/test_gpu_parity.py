@@ -614,7 +614,10 @@ def test_layernorm_backward_shapes_without_two_call_form(ops):
 
 
 @pytest.mark.parametrize("N,V,stride,dtype,grad_dtype", [
-    (512, 50257, 50304, torch.bfloat16, torch.bfloat16),   # the GPT-2 vocabulary, padded stride
+    (512, 50257, 50304, torch.bfloat16, torch.bfloat16),   # the GPT-2 vocabulary, padded stride: the streaming kernel
+    (300, 50257, 50304, torch.bfloat16, torch.float32),    # the same under the autocast rule
+    (200, 32000, 32000, torch.float16, torch.float16),     # streaming kernel, four vectors per lane
+    (96, 30000, 30000, torch.float32, torch.float32),      # streaming kernel, fp32 rows
     (300, 50257, 50257, torch.bfloat16, torch.float32),    # unpadded rows, the autocast combination
     (1024, 384, 384, torch.float32, torch.float32),        # the reference's test width
     (77, 1000, 1003, torch.float16, torch.float16),
