@@ -49,7 +49,7 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # algorithmic bytes per fused-classifier call: read the class columns of the logits once and
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
-CE_ROWS_TRAFFIC_BYTES = 1_650_508_000  # measured with rocprofv3 --pmc, see profiles/
+CE_ROWS_TRAFFIC_BYTES = 1_650_380_000  # measured with rocprofv3 --pmc (profiles/ce_rows_stream_kernel_hbm_traffic_pmc.txt)
 
 
 def log(*a):
@@ -1008,7 +1008,7 @@ def result_line(args, head, value, achieved, cpu, table):
         "per_op": compact_per_op(table),
         "roofline": {
             "bound": "hbm",
-            "kernel": "ce_rows_stream_kernel<bf16_t, bf16_t, 7, 8>",
+            "kernel": "ce_rows_stream_kernel<bf16_t, bf16_t, 7, 8, false>",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
