@@ -518,6 +518,30 @@ def test_adamw_all_parameters_in_one_task(host, sched, co):
     assert_bit_exact(down(host, sched, ws[1]), before, "skipped update")
 
 
+@pytest.mark.gpu
+def test_adamw_descriptor_tables_are_reused_only_when_identical(host, sched, co):
+    # the optimizer task keeps its last few descriptor tables on the device and skips the copy when
+    # a new table matches one byte for byte; ten different parameter sets stepped in turn (more than
+    # are kept) and the first set again must each get their own update
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    sets = []
+    for k in range(10):
+        w0 = [randn((64 + k, 8), 900 + k, std=0.02), randn((33,), 920 + k, std=0.02)]
+        g = [randn((64 + k, 8), 940 + k, std=1e-2), randn((33,), 960 + k, std=1e-2)]
+        ws = [up(host, sched, w) for w in w0]
+        gs = [up(host, sched, x) for x in g]
+        sets.append((w0, g, ws, gs, [host.AdamW.init(sched, w, **hp) for w in ws]))
+    for rnd in range(3):
+        for w0, g, ws, gs, states in sets:
+            host.AdamW.step_all(sched, states, ws, gs)
+    for w0, g, ws, gs, states in sets:
+        for i in range(2):
+            w, m, v = w0[i], torch.zeros_like(w0[i]), torch.zeros_like(w0[i])
+            for t in range(1, 4):
+                w, m, v, _ = co.adamw_step(w, g[i], m, v, t=t, **hp)
+            assert_close(down(host, sched, ws[i]), w.reshape(w0[i].shape), atol=1e-8, name="w")
+
+
 # ------------------------------------------------------------------- module layer
 def build_tree(host, sched, V=211, T=16, C=64):
     """A GPT-2-shaped tree: wte, wpe, h.0.ln_1, h.0.ln_2, ln_f (what the ops here cover)."""
