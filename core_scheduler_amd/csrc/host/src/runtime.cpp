@@ -187,6 +187,9 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
   }
 
   void submit(Task &&task) override {
+    // one submission at a time: the lanes' bookkeeping below is not shared between threads
+    // otherwise (the reference's submit is a push into a locked queue)
+    std::lock_guard<std::recursive_mutex> lock{submit_mutex_};
     c10::hip::HIPGuardMasqueradingAsCUDA device_guard{static_cast<c10::DeviceIndex>(device_rank_)};
     const auto &body = *task.impl();
     if (body.type() == Task::Impl::kConfig) {
@@ -322,6 +325,7 @@ struct ThreeStreamScheduler final : Scheduler::Impl {
     return keep;
   }
 
+  std::recursive_mutex submit_mutex_;  // recursive: a body may submit a task of its own
   std::vector<Stream> streams_;
   // per waiting lane and recording stream: position (Event::Impl::order) of the latest event that
   // the waiting lane's stream has been made to wait for, or has seen completed
