@@ -57,6 +57,9 @@ struct Event::Impl {
   }
   void settle() {
     if (!owed) return;
+    static auto *mutex = new std::mutex;  // a waiting thread and a submitting one may both get here
+    std::lock_guard<std::mutex> lock{*mutex};
+    if (!owed) return;
     c10::hip::HIPStreamGuardMasqueradingAsCUDA guard{*home};
     record();
   }
