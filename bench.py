@@ -969,11 +969,21 @@ def main():
 MAX_LINE_BYTES = 8000  # the result line on stdout stays below this; the full table goes to stderr
 
 
+# Rows that time an alternative way of issuing an op (the reference's two-stream LayerNorm
+# backward, a separate add launch, one AdamW launch per tensor) next to the library's own way.
+# They are in the full table, under their own names; the result line carries the ops themselves.
+COMPARISON_ROWS = ("layernorm_bwd_two_streams", "add_then_layernorm_fwd", "layernorm_bwd_then_add",
+                   "adamw_per_tensor_launches")
+
+
 def compact_per_op(table):
     """One short record per row of the per-op table: op, configuration tag, cold ms per call,
-    cold fraction of the HBM peak.  Everything else a row carries is in the full table."""
+    cold fraction of the HBM peak.  Everything else a row carries is in the full table, and so
+    are the comparison rows."""
     out = []
     for rec in table:
+        if rec["op"] in COMPARISON_ROWS:
+            continue
         parts = rec["config"].split(":")[0].split(", ")
         cfg = ", ".join(parts[:2]) if rec["op"] == "fused_classifier_call" else parts[0]
         out.append({"op": rec["op"], "cfg": cfg[:44], "ms": rec["ms_cold"], "frac": rec["frac_cold"]})
@@ -986,7 +996,7 @@ def result_line(args, head, value, achieved, cpu, table):
     line = {
         "metric": "per-op HBM GB/s (% of MI355X peak); fused CE ms at 8192x50257 bf16",
         "metric_note": "value = the fused classifier's whole-step GB/s (the ms is ms_per_step); every other op is in per_op "
-                       "(ms and fraction of the HBM peak per call, cold buffers); the full table is on stderr after [bench-full]",
+                       "(ms and fraction of the HBM peak per call, cold buffers); the full table, with rows that time alternative ways of issuing an op, is on stderr after [bench-full]",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
