@@ -332,7 +332,11 @@ __global__ __launch_bounds__(1024) void ce_rows_stream_kernel(
     scale0 = HAS_W ? dloss / reinterpret_cast<const float *>(ws_count)[1] : dloss / (float)(*ws_count);
   const float log2_scale0 = __builtin_amdgcn_logf(fabsf(scale0));  // -inf for 0: every output 0
 
-  int64_t row = blockIdx.x;
+  // Workgroups go round the eight XCDs in launch order.  The workgroups of one XCD take
+  // neighbouring rows of each round of gridDim rows (XCD 0 the first eighth, and so on) rather
+  // than every eighth row: [8192,50257] bf16 282.7 us per call against 285.2, with fp32 gradients
+  // 444.5 against 450.8.
+  int64_t row = (gridDim.x % 8 == 0) ? (int64_t)(blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
   VecE<T, EPV> cur[VPT];
   int64_t tgt = 0;
   bool live = false;
