@@ -49,7 +49,7 @@ CE_N, CE_V, CE_STRIDE = 8192, 50257, 50304
 # algorithmic bytes per fused-classifier call: read the class columns of the logits once and
 # write them once (bf16), read the int64 targets, write fp32 row losses and the mean
 CE_BYTES = 2 * CE_N * CE_V * 2 + CE_N * 8 + CE_N * 4 + 4
-CE_ROWS_TRAFFIC_BYTES = 1_650_380_000  # measured with rocprofv3 --pmc (profiles/ce_rows_stream_kernel_hbm_traffic_pmc.txt)
+CE_ROWS_TRAFFIC_BYTES = 1_649_121_000  # measured with rocprofv3 --pmc (profiles/ce_rows_stream_kernel_hbm_traffic_pmc.txt)
 
 
 def log(*a):
