@@ -29,6 +29,7 @@
 extern "C" {
 #endif
 
+/* raised when an existing entry point changes its arguments or meaning; new entry points leave it */
 #define CS_HIP_ABI_VERSION 1
 
 /* element types */
